@@ -97,6 +97,9 @@ def run_case(name, cache_size, static_size, B, D, prefill_lens, S, n_decode, use
 cases = []
 # the reference's own demo (cache_utils.py:1301-1371): left-padded rows 14, 9, 5
 cases.append(run_case("reference_demo", [5, 10], [2, 3], 3, 4, [14, 9, 5], 14, 9, True))
+# a left-padded row whose valid tokens do not fill its static part: the reference then
+# enters the ring early because its token counter includes padding (cache_utils.py:1041-1045,1139)
+cases.append(run_case("padded_short_row", [5, 10], [2, 3], 3, 4, [12, 2, 1], 12, 8, True))
 # same sizes, no mask
 cases.append(run_case("demo_no_mask", [5, 10], [2, 3], 3, 4, [14, 14, 14], 14, 9, False))
 # prompt shorter than static part of one head, then decode through the static->ring switch
