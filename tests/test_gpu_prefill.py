@@ -1,0 +1,205 @@
+"""GPU parity of the block-sparse prefill kernel (mixture_of_sparse_attention ->
+moa_prefill -> ctypes -> libmoa_hip.so) against the CPU oracle's dense masked
+attention in fp32.
+
+Tolerance (fp32 accumulate, P rounded to the input dtype before PV as in the
+reference kernel, output rounded to the input dtype):
+  fp16:  |out - oracle| <= 2e-3 + 1e-2 * |oracle|   -- the bound BASELINE states,
+         applied the way the reference's tests apply theirs (assert_close);
+  bf16:  |out - oracle| <= 1.6e-2 + 1e-2 * |oracle| -- same relative term; the
+         absolute term is scaled by 8 = 2^(11-8), the ratio of the two formats'
+         unit roundoffs, because the softmax weights enter the PV product
+         rounded to 8 significant bits (error up to 2^-9 * sum_i w_i |v_i|, which a
+         bound relative to |oracle| cannot absorb where the sum cancels).  The
+         reference has no bf16 prefill to compare with (its kernel asserts fp16,
+         MoA/kernels/block_sparse_attention_prefill.py:645-646)."""
+import warnings
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle.moa_oracle import moa_token_mask, prefill_masked_dense
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 2e-3, 1e-2
+ATOL_BF16 = 1.6e-2
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from moa_amd import _lib
+    _lib.load()
+    return torch.device("cuda:0")
+
+
+def _close(out, ref, tag):
+    atol = ATOL_BF16 if out.dtype == torch.bfloat16 else ATOL
+    out = out.float().cpu()
+    ref = ref.float().cpu()
+    assert torch.isfinite(out).all(), tag
+    err = (out - ref).abs()
+    bound = atol + RTOL * ref.abs()
+    bad = err > bound
+    assert not bad.any(), (tag, float(err.max()), int(bad.sum()), [int(x) for x in bad.nonzero()[0]])
+
+
+def _qkv(B, H, N, D, dtype, dev, seed, hkv=None):
+    g = torch.Generator().manual_seed(seed)
+    hkv = hkv or H
+    # projections come out as [B, N, H, D]; the operator gets [B, H, N, D] views of them
+    q = torch.randn(B, N, H, D, generator=g).to(dev, dtype).transpose(1, 2)
+    k = torch.randn(B, N, hkv, D, generator=g).to(dev, dtype).transpose(1, 2)
+    v = torch.randn(B, N, hkv, D, generator=g).to(dev, dtype).transpose(1, 2)
+    return q, k, v
+
+
+def _run(q, k, v, sm, ns, nl, dev):
+    from moa_amd import mixture_of_sparse_attention
+    H = k.shape[1]
+    sink = torch.tensor([x * 64 for x in ns], dtype=torch.int64, device=dev)
+    local = torch.tensor([x * 64 for x in nl], dtype=torch.int64, device=dev)
+    out = mixture_of_sparse_attention(q, k, v, sm, sink_size=sink, local_size=local)
+    B, Hq, N, D = q.shape
+    assert out.shape == (B, N, Hq, D) and out.dtype == q.dtype and out.is_contiguous()
+    return out.transpose(1, 2)   # [B,H,N,D] like the oracle
+
+
+def test_reference_prefill_test(dev):
+    """The reference's own prefill test (tests/attention_kernel_test.py:35-76):
+    uniform [0,1) fp16 data, B=2, H=4, N=128, D=128, sm_scale 0.1, sink 64 + local 64
+    (dense causal), "sdpa" against "moa" at rtol = atol = 1e-3, output [B, N, H, D]."""
+    from moa_amd import mixture_of_sparse_attention
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.rand(2, 4, 128, 128, generator=g).to(dev, torch.float16) for _ in range(3))
+    sink = torch.full((4,), 64, dtype=torch.int64, device=dev)
+    local = torch.full((4,), 64, dtype=torch.int64, device=dev)
+    out = {}
+    for impl in ("sdpa", "moa"):
+        out[impl] = mixture_of_sparse_attention(q, k, v, 0.1, attention_dropout=0.0, implementation=impl,
+                                                local_size=local, sink_size=sink)
+        assert out[impl].shape == (2, 128, 4, 128)
+    torch.testing.assert_close(out["sdpa"], out["moa"], rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("N", [64 * 5, 200, 333, 1000, 128, 65])
+def test_small_against_oracle(dev, dtype, D, N):
+    H = 6
+    ns = [1, 0, 2, 1, 0, 3]
+    nl = [2, 1, 1, 0, 3, 5]
+    q, k, v = _qkv(2, H, N, D, dtype, dev, seed=N + D)
+    sm = D ** -0.5
+    out = _run(q, k, v, sm, ns, nl, dev)
+    ref = prefill_masked_dense(q, k, v, sm, ns, nl)
+    _close(out, ref, (dtype, D, N))
+
+
+def test_dead_rows_are_zero(dev):
+    """ns = nl = 0 sees nothing; nl = 0 with sinks sees only sink blocks."""
+    q, k, v = _qkv(1, 2, 256, 128, torch.float16, dev, seed=3)
+    out = _run(q, k, v, 0.1, [0, 1], [0, 0], dev)
+    assert not out[:, 0].any()
+    ref = prefill_masked_dense(q, k, v, 0.1, [0, 1], [0, 0])
+    _close(out, ref, "dead")
+
+
+def test_wide_windows_reduce_to_causal(dev):
+    q, k, v = _qkv(1, 3, 1024, 128, torch.bfloat16, dev, seed=4)
+    out = _run(q, k, v, 128 ** -0.5, [0, 16, 1], [16, 0, 99], dev)
+    ref = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=True, scale=128 ** -0.5)
+    _close(out, ref, "causal")
+
+
+def test_gqa(dev):
+    """8 query heads on 2 kv heads: equals MHA with each kv head repeated 4 times."""
+    q, k, v = _qkv(2, 8, 448, 128, torch.float16, dev, seed=5, hkv=2)
+    ns, nl = [1, 2], [2, 3]
+    out = _run(q, k, v, 0.09, ns, nl, dev)
+    kr, vr = k.repeat_interleave(4, dim=1), v.repeat_interleave(4, dim=1)
+    ref = prefill_masked_dense(q, kr, vr, 0.09, [1] * 4 + [2] * 4, [2] * 4 + [3] * 4)
+    _close(out, ref, "gqa")
+
+
+def test_short_prompt_falls_back_to_dense(dev):
+    """N <= 64: dense causal with a warning (mixture_of_attention.py:412-415), whatever the spans."""
+    from moa_amd import mixture_of_sparse_attention
+    q, k, v = _qkv(2, 3, 40, 64, torch.float16, dev, seed=6)
+    with warnings.catch_warnings(record=True) as w:
+        warnings.simplefilter("always")
+        out = mixture_of_sparse_attention(q, k, v, 0.125)
+        assert any("Falling back to dense" in str(x.message) for x in w)
+    ref = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=True, scale=0.125)
+    _close(out.transpose(1, 2), ref, "short")
+
+
+def test_invariants(dev):
+    q, k, v = _qkv(2, 4, 704, 128, torch.float16, dev, seed=7)
+    ns, nl = [1, 1, 0, 2], [3, 1, 4, 2]
+    out = _run(q, k, v, 0.09, ns, nl, dev)
+    ones = _run(q, k, torch.ones_like(v), 0.09, ns, nl, dev)
+    assert (ones.float() - 1).abs().max().item() <= 1e-3
+    perm = [2, 0, 3, 1]
+    outp = _run(q[:, perm], k[:, perm], v[:, perm], 0.09, [ns[i] for i in perm], [nl[i] for i in perm], dev)
+    assert torch.equal(outp, out[:, perm])
+    outb = _run(q[1:], k[1:], v[1:], 0.09, ns, nl, dev)
+    assert torch.equal(outb, out[1:])
+
+
+def test_cpu_reference_config(dev):
+    """BASELINE configs[0]: one layer, 32 heads, head_dim 64, batch 1, seq 2048, 64 sinks,
+    per-head window from {256,...,1024}; inputs N(0,1).  The GPU path runs it in
+    fp16 (the config's fp32 is the oracle's arithmetic); whole output against the oracle."""
+    from moa_amd.workloads import uniform_block_windows
+    B, H, N, D = 1, 32, 2048, 64
+    q, k, v = _qkv(B, H, N, D, torch.float16, dev, seed=0)
+    win = uniform_block_windows(H, seed=0)
+    ns, nl = [1] * H, [w // 64 for w in win]
+    sm = D ** -0.5
+    out = _run(q, k, v, sm, ns, nl, dev)
+    ref = prefill_masked_dense(q, k, v, sm, ns, nl)
+    _close(out, ref, "C1")
+
+
+def test_prefill_config_scale(dev):
+    """BASELINE configs[1] at full size (B=4, H=32, D=128, N=8192, bf16, elastic spans):
+    (a) V == 1 => O == 1 everywhere; (b) three whole heads against the CPU oracle;
+    (c) one batch element against torch's dense masked attention in fp32 on the GPU."""
+    from moa_amd.workloads import elastic_spans
+    B, H, N, D = 4, 32, 8192, 128
+    q, k, v = _qkv(B, H, N, D, torch.bfloat16, dev, seed=1)
+    spans = elastic_spans(H, N, seed=0)
+    ns, nl = [1] * H, [s // 64 for s in spans]
+    sm = D ** -0.5
+    out = _run(q, k, v, sm, ns, nl, dev)
+    ones = _run(q, k, torch.ones_like(v), sm, ns, nl, dev)
+    assert (ones.float() - 1).abs().max().item() <= 8e-3   # bf16 output spacing near 1
+    for b, h in [(0, int(np.argmin(nl))), (3, int(np.argmax(nl))), (2, 17)]:
+        ref = prefill_masked_dense(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], sm,
+                                   [ns[h]], [nl[h]])
+        _close(out[b:b + 1, h:h + 1], ref, (b, h))
+    b = 1
+    for h0 in range(0, H, 8):
+        mask = torch.stack([torch.from_numpy(moa_token_mask(N, ns[h], nl[h])) for h in range(h0, h0 + 8)]).to(dev)
+        ref = F.scaled_dot_product_attention(q[b:b + 1, h0:h0 + 8].float(), k[b:b + 1, h0:h0 + 8].float(),
+                                             v[b:b + 1, h0:h0 + 8].float(), attn_mask=mask[None], scale=sm)
+        _close(out[b:b + 1, h0:h0 + 8], ref, ("gpu dense", h0))
+
+
+def test_errors(dev):
+    from moa_amd import mixture_of_sparse_attention
+    q = torch.zeros(1, 2, 128, 128, dtype=torch.float32, device=dev)
+    s = torch.tensor([64, 64], device=dev)
+    with pytest.raises(AssertionError):   # fp32 (reference: block_sparse_attention_prefill.py:645-646)
+        mixture_of_sparse_attention(q, q, q, 1.0, sink_size=s, local_size=s)
+    q96 = torch.zeros(1, 2, 128, 96, dtype=torch.float16, device=dev)
+    with pytest.raises(NotImplementedError):
+        mixture_of_sparse_attention(q96, q96, q96, 1.0, sink_size=s, local_size=s)
+    qa = torch.zeros(1, 2, 128, 128, dtype=torch.float16, device=dev)
+    kb = torch.zeros(1, 2, 128, 64, dtype=torch.float16, device=dev)
+    with pytest.raises(AssertionError):
+        mixture_of_sparse_attention(qa, kb, qa, 1.0, sink_size=s, local_size=s)
