@@ -46,6 +46,8 @@ def parse_args():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--prefill-iters", type=int, default=10)
+    ap.add_argument("--only", choices=["decode", "prefill"], default=None,
+                    help="profiling aid: run one part only and print its figures (not the contract line)")
     return ap.parse_args()
 
 
@@ -247,8 +249,14 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.only == "prefill":
+        print(json.dumps({"prefill": bench_prefill(torch, dev, args)}))
+        return
     dec = bench_decode(torch, dev, args)
     del dec["cache"]
+    if args.only == "decode":
+        print(json.dumps({"decode": dec}))
+        return
     torch.cuda.empty_cache()
     pre = None
     if not args.no_prefill:
