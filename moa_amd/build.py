@@ -28,6 +28,8 @@ HIPCC_FLAGS = [
     "-fno-gpu-rdc",
     "-Wall",
     "-Wno-unused-function",
+    # no kernel relies on NaN propagation (masks use -inf): lets fmax compile to one instruction
+    "-fno-honor-nans",
     # packed-FP32 instructions are switched off for all device code of this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
@@ -52,7 +54,8 @@ def is_stale() -> bool:
 
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    extra = os.environ.get("MOA_HIPCC_FLAGS", "").split()   # e.g. -DNAME for an experiment build
+    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")

@@ -13,8 +13,12 @@
 //     query blocks of one (batch, head); each wave owns 32 rows;
 //   * it walks the union of the live 64-key tiles of its two query blocks; a
 //     wave skips the MFMA work of a tile that is dead for ITS query block;
-//   * K and V tiles go global -> registers -> LDS (row-major, padded rows);
-//     the next tile's global loads are issued before the current tile's math.
+//   * K and V tiles go global -> registers -> LDS (row-major, padded rows,
+//     two buffers each): the next tile's global loads are issued one
+//     iteration ahead and written to the other buffer after this tile's math,
+//     so there is one work-group barrier per tile;
+//   * the LDS reads of the MFMA operands are issued several MFMAs ahead of
+//     their use.
 //
 // Matrix layout.  Both GEMMs are computed transposed so that every per-row
 // softmax quantity lives in ONE lane:
@@ -98,9 +102,14 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_kernel(
   constexpr int CPR = D / 8;          // 16-byte chunks per row
   constexpr int RPP = kPfThreads / CPR;   // rows per pass of the cooperative tile load
   constexpr int PASSES = kKV / RPP;
+  constexpr int KTILE = kKV * LDK;    // elements of one K buffer
+  constexpr int VTILE = kKV * LDV;
+  constexpr float kRescaleStep = 8.f; // rescale O only when a row max grew by more than 2^8
 
-  __shared__ __attribute__((aligned(16))) uint16_t s_k[kKV * LDK];
-  __shared__ __attribute__((aligned(16))) uint16_t s_v[kKV * LDV];
+  // two K and two V buffers: tile j+1 is written while tile j is being read
+  extern __shared__ __attribute__((aligned(16))) uint16_t s_mem[];
+  uint16_t* const s_k = s_mem;
+  uint16_t* const s_v = s_mem + 2 * KTILE;
 
   // ---- which (head, query tile) --------------------------------------------
   // Work-groups are dealt to the 8 XCDs round-robin by the hardware.  Group
@@ -119,13 +128,13 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_kernel(
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int mcol = lane & 31;   // query row inside the wave's 32 (the MFMA column)
   const int g = lane >> 5;      // half-wave
 
   const int nb = (N + kKV - 1) / kKV;
-  const int ns = (int)sink_blocks[hk];
-  const int nl = (int)local_blocks[hk];
+  const int ns = __builtin_amdgcn_readfirstlane((int)sink_blocks[hk]);
+  const int nl = __builtin_amdgcn_readfirstlane((int)local_blocks[hk]);
   const int mb0 = 2 * qt;                                  // first query block of the group
   const int mb1 = min(2 * qt + 1, nb - 1);                 // last one that exists
   const int mbw = 2 * qt + (wave >> 1);                    // this wave's query block
@@ -158,67 +167,108 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_kernel(
   for (int t = 0; t < DT; ++t)
 #pragma unroll
     for (int i = 0; i < 16; ++i) oacc[t][i] = 0.f;
-  float m_run = -INFINITY;   // running max of scale_log2 * s
+  float m_run = -INFINITY;   // reference max of scale_log2 * s used by exp2 (lags the true max by <= kRescaleStep)
   float l_run = 0.f;         // this lane's share of the running sum (the lane+32 twin holds the rest)
 
   // ---- cooperative tile load: thread -> (row, 16-byte chunk) ----------------
   const int ld_row = tid / CPR;
   const int ld_chk = tid % CPR;
-  const uint16_t* kbase = k + b * ks.b + hk * ks.h + ld_chk * 8;
-  const uint16_t* vbase = v + b * vs.b + hk * vs.h + ld_chk * 8;
+  const uint16_t* kbase = k + b * ks.b + hk * ks.h;   // uniform
+  const uint16_t* vbase = v + b * vs.b + hk * vs.h;
+  uint32_t koff[PASSES], voff[PASSES];                // element offsets inside a tile
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    koff[p] = (uint32_t)((p * RPP + ld_row) * ks.n + ld_chk * 8);
+    voff[p] = (uint32_t)((p * RPP + ld_row) * vs.n + ld_chk * 8);
+  }
   u32x4 kreg[PASSES], vreg[PASSES];
 
   auto issue_loads = [&](int j) {
+    const uint16_t* kt = kbase + (int64_t)j * kKV * ks.n;
+    const uint16_t* vt = vbase + (int64_t)j * kKV * vs.n;
+    if ((j + 1) * kKV <= N) {
+#pragma unroll
+      for (int p = 0; p < PASSES; ++p) {
+        kreg[p] = *reinterpret_cast<const u32x4*>(kt + koff[p]);
+        vreg[p] = *reinterpret_cast<const u32x4*>(vt + voff[p]);
+      }
+    } else {   // the ragged last tile: rows >= N read as zero
+#pragma unroll
+      for (int p = 0; p < PASSES; ++p) {
+        const bool ok = j * kKV + p * RPP + ld_row < N;
+        u32x4 z = {0, 0, 0, 0};
+        kreg[p] = ok ? *reinterpret_cast<const u32x4*>(kt + koff[p]) : z;
+        vreg[p] = ok ? *reinterpret_cast<const u32x4*>(vt + voff[p]) : z;
+      }
+    }
+  };
+  auto store_tile = [&](int buf) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
-      const int64_t n = (int64_t)j * kKV + p * RPP + ld_row;
-      u32x4 z = {0, 0, 0, 0};
-      const bool ok = n < N;
-      kreg[p] = ok ? *reinterpret_cast<const u32x4*>(kbase + n * ks.n) : z;
-      vreg[p] = ok ? *reinterpret_cast<const u32x4*>(vbase + n * vs.n) : z;
+      const int r = p * RPP + ld_row;
+      *reinterpret_cast<u32x4*>(s_k + buf * KTILE + r * LDK + ld_chk * 8) = kreg[p];
+      *reinterpret_cast<u32x4*>(s_v + buf * VTILE + r * LDV + ld_chk * 8) = vreg[p];
     }
   };
   auto next_tile = [&](int j) { return (j == hi1) ? lo2 : j + 1; };
 
-  int j = (hi1 >= 0) ? 0 : lo2;
-  if (j <= mb1) issue_loads(j);
-
-  // operand read positions
-  const uint16_t* k_rd = s_k + mcol * LDK + 8 * g;                       // + 32*nt*LDK + 16*ks
+  // operand read positions inside a buffer
+  const int k_rd_off = mcol * LDK + 8 * g;                               // + 32*nt*LDK + 16*ks
   const int grp16 = lane & 15;
   const int dhalf = (lane >> 4) & 1;
-  const uint16_t* v_rd = s_v + (4 * g + (grp16 >> 2)) * LDV + 16 * dhalf + 4 * (grp16 & 3);
+  const int v_rd_off = (4 * g + (grp16 >> 2)) * LDV + 16 * dhalf + 4 * (grp16 & 3);
                                                                          // + (16*t [+8])*LDV + 32*dt
 
-  while (j <= mb1) {
-    __syncthreads();   // everyone is done reading the previous tile
+  int j = (hi1 >= 0) ? 0 : lo2;
+  if (j > mb1) {   // nothing is visible from this query tile: zeros
+    if (wave_has_rows && m_glob < N) {
+      uint16_t* orow = o + b * os.b + hq * os.h + m_glob * os.n;
+      u32x2 z = {0, 0};
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const int r = p * RPP + ld_row;
-      *reinterpret_cast<u32x4*>(s_k + r * LDK + ld_chk * 8) = kreg[p];
-      *reinterpret_cast<u32x4*>(s_v + r * LDV + ld_chk * 8) = vreg[p];
+      for (int i = 0; i < D / 8; ++i) *reinterpret_cast<u32x2*>(orow + 8 * i + 4 * g) = z;
     }
-    __syncthreads();
-    const int jn = next_tile(j);
-    if (jn <= mb1) issue_loads(jn);
+    return;
+  }
+  issue_loads(j);
+  store_tile(0);
+  int jn = next_tile(j);
+  if (jn <= mb1) issue_loads(jn);
+  __syncthreads();
 
+  int buf = 0;
+  while (true) {
     const bool live = wave_has_rows && (j <= w_hi1 || (j >= w_lo2 && j <= mbw));
     if (live) {
-      // ---- S^T = K Q^T : two 32-key tiles ----
+      const uint16_t* k_rd = s_k + buf * KTILE + k_rd_off;
+      const uint16_t* v_rd = s_v + buf * VTILE + v_rd_off;
+      // ---- S^T = K Q^T : two 32-key tiles; the operand reads run kPre MFMAs ahead ----
       f32x16 st[2];
+      {
+        constexpr int kPre = 8;
+        u32x4 a[2 * KS];
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
+        for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) st[nt][i] = 0.f;
+          for (int s = 0; s < KS; ++s)
+            a[nt * KS + s] = *reinterpret_cast<const u32x4*>(k_rd + nt * 32 * LDK + 16 * s);
 #pragma unroll
-        for (int s = 0; s < KS; ++s) {
-          const u32x4 a = *reinterpret_cast<const u32x4*>(k_rd + nt * 32 * LDK + 16 * s);
-          st[nt] = T::mfma(a, qf[s], st[nt]);
+        for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) st[nt][i] = 0.f;
+#pragma unroll
+          for (int s = 0; s < KS; ++s) st[nt] = T::mfma(a[nt * KS + s], qf[s], st[nt]);
         }
+        __builtin_amdgcn_sched_group_barrier(0x100, kPre < 2 * KS ? kPre : 2 * KS, 0);
+#pragma unroll
+        for (int i = 0; i < 2 * KS - kPre; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, kPre < 2 * KS ? kPre : 2 * KS, 0);
       }
       // ---- causal mask on the diagonal tile ----
       if (j == mbw) {
-        const int m_in = wave * kWRows + mcol - (wave >> 1) * kKV;   // row inside the 64-row block
+        const int m_in = (wave & 1) * kWRows + mcol;   // row inside the 64-row block
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
@@ -227,46 +277,74 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_kernel(
             if (n_in > m_in) st[nt][i] = -INFINITY;
           }
       }
-      // ---- online softmax, base 2 ----
+      // ---- online softmax, base 2, with a lagging reference max ----
       float mx = st[0][0];
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) mx = fmaxf(mx, st[nt][i]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run, mx * scale_log2);   // finite: a live tile has a visible key in every row
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      const float m_cand = mx * scale_log2;   // finite: a live tile has a visible key in every row
+      // exp2 arguments stay <= kRescaleStep as long as no row max outgrew its reference by more
+      // than that; only then are O and l rescaled (a wave-uniform, rare branch after the first tile)
+      if (__any(m_cand > m_run + kRescaleStep)) {
+        const float m_new = fmaxf(m_run, m_cand);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        l_run *= alpha;
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) oacc[t][i] *= alpha;
+        m_run = m_new;
+      }
       float psum = 0.f;
       uint32_t pf[16];
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int i = 0; i < 16; i += 2) {
-          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i], scale_log2, -m_new));
-          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i + 1], scale_log2, -m_new));
+          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i], scale_log2, -m_run));
+          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i + 1], scale_log2, -m_run));
           psum += p0 + p1;
           pf[nt * 8 + (i >> 1)] = T::pack(p0, p1);
         }
-      l_run = l_run * alpha + psum;
-      m_run = m_new;
+      l_run += psum;
+      // ---- O^T += V^T P^T ; operand reads run kPre MFMAs ahead ----
+      {
+        constexpr int kPre = 4;
+        u32x4 a[4 * DT];
 #pragma unroll
-      for (int t = 0; t < DT; ++t)
+        for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) oacc[t][i] *= alpha;
-      // ---- O^T += V^T P^T ----
+          for (int dt = 0; dt < DT; ++dt) {
+            const u32x2 lo = lds_read_tr16(v_rd + (16 * t) * LDV + 32 * dt);
+            const u32x2 hi = lds_read_tr16(v_rd + (16 * t + 8) * LDV + 32 * dt);
+            a[t * DT + dt] = u32x4{lo.x, lo.y, hi.x, hi.y};
+          }
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const u32x4 bfrag = {pf[4 * t], pf[4 * t + 1], pf[4 * t + 2], pf[4 * t + 3]};
+        for (int t = 0; t < 4; ++t) {
+          const u32x4 bfrag = {pf[4 * t], pf[4 * t + 1], pf[4 * t + 2], pf[4 * t + 3]};
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          const u32x2 lo = lds_read_tr16(v_rd + (16 * t) * LDV + 32 * dt);
-          const u32x2 hi = lds_read_tr16(v_rd + (16 * t + 8) * LDV + 32 * dt);
-          const u32x4 a = {lo.x, lo.y, hi.x, hi.y};
-          oacc[dt] = T::mfma(a, bfrag, oacc[dt]);
+          for (int dt = 0; dt < DT; ++dt) oacc[dt] = T::mfma(a[t * DT + dt], bfrag, oacc[dt]);
         }
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * kPre, 0);
+#pragma unroll
+        for (int i = 0; i < 4 * DT - kPre; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, kPre, 0);
       }
     }
+    if (jn > mb1) break;
+    // tile jn (in registers since the previous iteration) goes into the other buffer; every wave
+    // left that buffer before the last barrier
+    store_tile(buf ^ 1);
     j = jn;
+    jn = next_tile(j);
+    if (jn <= mb1) issue_loads(jn);
+    __syncthreads();
+    buf ^= 1;
   }
 
   // ---- epilogue: O[m][d] = O^T[d][m] / l ---------------------------------
@@ -287,6 +365,11 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_kernel(
 }
 
 template <typename T, int D>
+static size_t prefill_lds_bytes() {
+  return (size_t)2 * kKV * ((D + 8) + (D + 32)) * sizeof(uint16_t);
+}
+
+template <typename T, int D>
 static int launch_prefill(const void* q, const void* k, const void* v, void* o, const int64_t* qs,
                           const int64_t* ks, const int64_t* vs, const int64_t* os, int B, int Hq,
                           int Hkv, int N, const int64_t* sink_blocks, const int64_t* local_blocks,
@@ -297,7 +380,17 @@ static int launch_prefill(const void* q, const void* k, const void* v, void* o, 
   if (groups > 0x7fffffffLL) return fail(MOA_ERR_UNSUPPORTED, "moa_prefill_fwd: too many work-groups");
   Strides4 sq = {qs[0], qs[1], qs[2]}, sk = {ks[0], ks[1], ks[2]}, sv = {vs[0], vs[1], vs[2]},
            so = {os[0], os[1], os[2]};
-  hipLaunchKernelGGL((prefill_kernel<T, D>), dim3((unsigned)groups), dim3(kPfThreads), 0, st,
+  const size_t lds = prefill_lds_bytes<T, D>();
+  static bool attr_set = false;   // per template instance
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_kernel<T, D>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess)
+      return fail(MOA_ERR_LAUNCH, "moa_prefill_fwd: cannot reserve %zu bytes of LDS: %s", lds,
+                  hipGetErrorString(e));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((prefill_kernel<T, D>), dim3((unsigned)groups), dim3(kPfThreads), lds, st,
                      (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (uint16_t*)o, sq, sk, sv,
                      so, BH, Hq, Hq / Hkv, N, n_qtiles, sink_blocks, local_blocks, sm_scale * kLog2eF);
   return check_launch("moa_prefill_fwd");
