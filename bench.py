@@ -32,6 +32,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+# HBM bytes moved by one decode launch divided by its algorithmic bytes, from two rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE) scaled by a 1 GiB copy kernel's readings; see
+# profiles/hbm_traffic_decode_and_prefill.txt.  bench.py cannot profile itself, so the ratio is carried here.
+DECODE_TRAFFIC_RATIO = 1.003
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense bf16 / fp16
 
 
@@ -46,7 +50,7 @@ def parse_args():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--prefill-iters", type=int, default=10)
-    ap.add_argument("--only", choices=["decode", "prefill"], default=None,
+    ap.add_argument("--only", choices=["decode", "prefill", "copy"], default=None,
                     help="profiling aid: run one part only and print its figures (not the contract line)")
     return ap.parse_args()
 
@@ -249,6 +253,17 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.only == "copy":
+        # calibration for the HBM traffic counters: a plain device copy of known size (1 GiB read,
+        # 1 GiB written per launch by torch's elementwise copy kernel)
+        n = 1 << 30
+        x = torch.empty(n, dtype=torch.uint8, device=dev).random_(0, 255)
+        y = torch.empty_like(x)
+        for _ in range(5):
+            y.copy_(x)
+        torch.cuda.synchronize(dev)
+        print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n, "launches": 5}))
+        return
     if args.only == "prefill":
         print(json.dumps({"prefill": bench_prefill(torch, dev, args)}))
         return
@@ -294,7 +309,9 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": dec["decode_gbs"] / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": DECODE_TRAFFIC_RATIO * dec["decode_bytes"],
+            "traffic_source": "profiles/hbm_traffic_decode_and_prefill.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
+                              "copy-kernel scaled; measured ratio to algorithmic bytes)",
             "bytes_per_launch": dec["decode_bytes"],
             "ms_per_launch": dec["decode_ms"],
         },

@@ -33,7 +33,10 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kDecThreads = 256;
 constexpr int kDecWaves = kDecThreads / 64;
-constexpr int kBatch = 8;          // wave-wide loads in flight per tensor
+#ifndef MOA_DEC_BATCH
+#define MOA_DEC_BATCH 8
+#endif
+constexpr int kBatch = MOA_DEC_BATCH;   // wave-wide loads in flight per tensor
 constexpr int kMaxHeads = 256;     // heads per batch row the LDS prefix covers
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -307,7 +310,13 @@ __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
   }
 }
 
-constexpr int kChunk = 512;
+#ifndef MOA_DEC_CHUNK
+#define MOA_DEC_CHUNK 512
+#endif
+#ifndef MOA_DEC_BLOCKS
+#define MOA_DEC_BLOCKS 16
+#endif
+constexpr int kChunk = MOA_DEC_CHUNK;
 
 static inline int64_t decode_cap(int64_t sumC, int H) { return (sumC + kChunk - 1) / kChunk + H; }
 
@@ -316,8 +325,9 @@ static int launch_decode(const void* q, const void* kc, const void* vc, void* o,
                          float* part_ml, const int64_t* head_start, const int64_t* head_valid, int B,
                          int H, int64_t sumC, float sm_scale, hipStream_t st) {
   const int cap = (int)decode_cap(sumC, H);
-  // enough blocks per batch row to fill 256 CUs several times over, never more than chunks exist
-  int bx = (int)((256 * 8 + B - 1) / B);
+  // 16 work-groups per CU over the whole grid (measured: 8 leaves a visible tail, 32 is no better),
+  // never more per batch row than chunks exist
+  int bx = (int)((256 * MOA_DEC_BLOCKS + B - 1) / B);
   if (bx > cap) bx = cap;
   if (bx < 1) bx = 1;
   hipLaunchKernelGGL((decode_split_kernel<T, D, kChunk>), dim3(bx, B), dim3(kDecThreads), 0, st,
