@@ -9,16 +9,17 @@
 // the causal test inside the diagonal block (:558-580).
 //
 // Work decomposition
-//   * one work-group (4 waves) owns 128 consecutive query rows = two 64-row
-//     query blocks of one (batch, head); each wave owns 32 rows;
-//   * it walks the union of the live 64-key tiles of its two query blocks; a
-//     wave skips the MFMA work of a tile that is dead for ITS query block;
-//   * K and V tiles go global -> registers -> LDS (row-major, padded rows,
-//     two buffers each): the next tile's global loads are issued one
-//     iteration ahead and written to the other buffer after this tile's math,
-//     so there is one work-group barrier per tile;
-//   * the LDS reads of the MFMA operands are issued several MFMAs ahead of
-//     their use.
+//   * one work-group of 8 waves owns 256 consecutive query rows (four 64-row
+//     query blocks) of one (batch, head); each wave owns 32 rows;
+//   * it walks the union of the live 64-key tiles of its four query blocks; a
+//     wave skips the math of a tile that is dead for ITS query block;
+//   * K and V tiles are copied global -> LDS asynchronously (no registers),
+//     four stages deep, rows unpadded with XOR-permuted 16-byte chunks so
+//     that every operand read is bank-conflict free;
+//   * the band of a work-group is walked circularly from the tile whose index is
+//     a multiple of the band length, so that neighbouring query tiles of a head
+//     (resident on one XCD at the same time) ask for the same tile at the same
+//     step and share it in L2.
 //
 // Matrix layout.  Both GEMMs are computed transposed so that every per-row
 // softmax quantity lives in ONE lane:
@@ -30,24 +31,34 @@
 // B-operand order (the contraction index n may be permuted freely as long as A
 // and B agree; the V^T operand is fetched with that same permutation by
 // ds_read_b64_tr_b16, which returns 4 consecutive rows of one column).
+//
+// Schedule.  A tile costs a wave 32 MFMAs (~1000 matrix-core cycles) and about
+// as many cycles of softmax VALU work, and the two do not overlap inside one
+// wave.  The 8 waves therefore run as two groups of four, one wave of each
+// group per SIMD.  Between two work-group barriers (one per tile) group A runs
+// its matrix phase (P.V of the previous tile, Q.K^T of the current one) and then
+// its softmax; group B, one phase behind, runs the softmax of the previous tile
+// and then its matrix phase, so each SIMD has one wave on the matrix pipe and
+// one on the vector ALU most of the time.  The matrix phase is free of VALU
+// instructions: operand addresses are kept per lane in registers, stage and row
+// selection go into the instructions' immediate offsets.
 #include "moa_common.h"
 
 namespace moa {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kPfThreads = 256;
-constexpr int kQRows = 128;   // query rows per work-group
+constexpr int kPfThreads = 512;
+constexpr int kQRows = 256;   // query rows per work-group
 constexpr int kWRows = 32;    // query rows per wave
 constexpr int kKV = 64;       // keys per tile (the sparsity block)
+constexpr int kStages = 4;    // LDS stages per tensor
 constexpr float kLog2eF = 1.4426950408889634f;
 
 struct PF16 {
@@ -63,6 +74,11 @@ struct PF16 {
     h2 r = {(_Float16)lo, (_Float16)hi};
     return __builtin_bit_cast(uint32_t, r);
   }
+  // acc + lo + hi of a packed pair (v_dot2_f32_f16 with a pair of ones)
+  static __device__ __forceinline__ float add_pair(uint32_t pk, float acc) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, pk), h2{(_Float16)1.f, (_Float16)1.f}, acc, false);
+  }
 };
 struct PBF16 {
   static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
@@ -74,42 +90,112 @@ struct PBF16 {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2v));
   }
   static __device__ __forceinline__ uint32_t pack_rne(float lo, float hi) { return pack(lo, hi); }
+  // acc + lo + hi of a packed pair (v_dot2_f32_bf16 with a pair of ones)
+  static __device__ __forceinline__ float add_pair(uint32_t pk, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2v, pk), __builtin_bit_cast(bf16x2v, 0x3f803f80u), acc, false);
+  }
 };
 
 // 4 consecutive rows of one 16-bit column out of a row-major LDS tile: within
 // each group of 16 lanes, lane i must point at (row0 + i/4, col0 + 4*(i%4));
 // it receives rows row0..row0+3 of column col0 + i.
-__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* p) {
+__device__ __forceinline__ u32x2 lds_read_tr16(const char* p) {
   typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
   s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
   return __builtin_bit_cast(u32x2, r);
 }
 
+// Asynchronous 16-byte-per-lane copy global -> LDS (global_load_lds_dwordx4): lane i of the wave
+// reads base + byte_off(i) and lands at LDS byte address lds_addr + 16*i.  base and lds_addr are
+// wave-uniform.  Written as inline assembly on purpose: the compiler cannot prove that these LDS
+// writes do not alias the operand reads of the stage being computed and would otherwise put a
+// full vmcnt(0) wait in front of every LDS read; completion is tracked by hand with wait_vm().
+// Loads complete in order, so the compiler's own vmcnt bookkeeping for ordinary loads stays safe
+// (it can only wait longer than it planned).
+__device__ __forceinline__ void async_copy16(const void* base, uint32_t byte_off, uint32_t lds_addr) {
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %0, %1"
+      :
+      : "v"(byte_off), "s"(base), "s"(__builtin_amdgcn_readfirstlane(lds_addr))
+      : "memory");
+}
+// max of a value with its twin in the other half of the wave (lane ^ 32), without going through LDS
+__device__ __forceinline__ float max_with_other_half(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ uint32_t lds_address(const char* p) {
+  return (uint32_t)(uintptr_t)((const char __attribute__((address_space(3)))*)p);
+}
+// Wait until at most n of this wave's global loads / async copies are outstanding.
+__device__ __forceinline__ void wait_vm(int n) {
+  if (n >= 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else if (n >= 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+  else if (n >= 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  else if (n == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+  else if (n == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+  else if (n == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// Work-group barrier WITHOUT the memory fence of __syncthreads(): the fence would make every wave
+// wait for all of its outstanding async copies (vmcnt(0)) at each phase boundary and serialise the
+// copy pipeline.  What must be visible at a barrier is waited for explicitly with wait_vm().
+__device__ __forceinline__ void phase_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+
+
 struct Strides4 {
   int64_t b, h, n;
 };
 
+template <int P>
+struct IC {
+  static constexpr int value = P;
+};
+
+// LDS accesses by 32-bit LDS byte address (a VGPR) plus a compile-time offset, so that the stage
+// and row selection of an operand costs no VALU instruction.
+__device__ __forceinline__ u32x4 lds_load16(uint32_t addr, int imm) {
+  typedef u32x4 __attribute__((address_space(3))) * lds_u32x4_ptr;
+  return *(lds_u32x4_ptr)(uintptr_t)(addr + imm);
+}
+__device__ __forceinline__ u32x2 lds_load_tr16(uint32_t addr, int imm) {
+  typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+  s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(uintptr_t)(addr + imm));
+  return __builtin_bit_cast(u32x2, r);
+}
+
 template <typename T, int D>
-__global__ __launch_bounds__(kPfThreads, 2) void prefill_kernel(
+__global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
     uint16_t* __restrict__ o, Strides4 qs, Strides4 ks, Strides4 vs, Strides4 os, int BH, int Hq,
     int group, int N, int n_qtiles, const int64_t* __restrict__ sink_blocks,
     const int64_t* __restrict__ local_blocks, float scale_log2) {
   constexpr int KS = D / 16;          // MFMA k-steps of the QK^T product
   constexpr int DT = D / 32;          // 32-wide d tiles of the output
-  constexpr int LDK = D + 8;          // K tile row stride (elements): rows shift 4 banks
-  constexpr int LDV = D + 32;         // V tile row stride: rows shift 16 banks
-  constexpr int CPR = D / 8;          // 16-byte chunks per row
-  constexpr int RPP = kPfThreads / CPR;   // rows per pass of the cooperative tile load
-  constexpr int PASSES = kKV / RPP;
-  constexpr int KTILE = kKV * LDK;    // elements of one K buffer
-  constexpr int VTILE = kKV * LDV;
+  constexpr int CPR = D / 8;          // 16-byte chunks per K/V row
+  constexpr int LPW = CPR / 8;        // async copies per wave per tile and tensor (64 chunks each)
+  constexpr int TILE_B = kKV * D * 2; // bytes of one K or V stage (rows unpadded)
+  constexpr int ROW_B = D * 2;
+  constexpr int RSH = 16 / CPR;       // rows per 256 bytes of LDS (1 at D=128, 2 at D=64)
   constexpr float kRescaleStep = 8.f; // rescale O only when a row max grew by more than 2^8
+  static_assert(4 * DT == 2 * KS, "P.V and Q.K^T have the same number of MFMAs per tile");
 
-  // two K and two V buffers: tile j+1 is written while tile j is being read
-  extern __shared__ __attribute__((aligned(16))) uint16_t s_mem[];
-  uint16_t* const s_k = s_mem;
-  uint16_t* const s_v = s_mem + 2 * KTILE;
+  // LDS: kStages K stages, then kStages V stages; tile t lives in stage t % kStages.  Rows are
+  // unpadded (an async copy fills 1 KiB of consecutive LDS) with their 16-byte chunks XOR-permuted:
+  //   K: chunk c of row n sits at position c ^ ((n / RSH) % CPR)           (16 rows x same chunk)
+  //   V: chunk c of row n sits at position c ^ (4 * ((n / RSH) % (CPR/4)))  (4 rows x 4 chunks)
+  extern __shared__ __attribute__((aligned(1024))) char s_mem[];
+  char* const s_k = s_mem;
+  char* const s_v = s_mem + kStages * TILE_B;
 
   // ---- which (head, query tile) --------------------------------------------
   // Work-groups are dealt to the 8 XCDs round-robin by the hardware.  Group
@@ -129,26 +215,97 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int grp = wave >> 2;    // 0: group A, 1: group B (one phase behind A)
   const int mcol = lane & 31;   // query row inside the wave's 32 (the MFMA column)
   const int g = lane >> 5;      // half-wave
 
   const int nb = (N + kKV - 1) / kKV;
   const int ns = __builtin_amdgcn_readfirstlane((int)sink_blocks[hk]);
   const int nl = __builtin_amdgcn_readfirstlane((int)local_blocks[hk]);
-  const int mb0 = 2 * qt;                                  // first query block of the group
-  const int mb1 = min(2 * qt + 1, nb - 1);                 // last one that exists
-  const int mbw = 2 * qt + (wave >> 1);                    // this wave's query block
+  const int mb0 = 4 * qt;                                  // first query block of the group
+  const int mbl = min(4 * qt + 3, nb - 1);                 // last one that exists
+  const int mbw = 4 * qt + (wave >> 1);                    // this wave's query block
   const bool wave_has_rows = mbw < nb;
 
-  // tile ranges of the work-group: sinks [0, hi1], then band [lo2, mb1]
-  const int hi1 = min(ns - 1, mb1);
+  // tiles of the work-group: sinks [0, hi1], then band [lo2, mbl]
+  const int hi1 = min(ns - 1, mbl);
   int lo2 = max(0, mb0 + 1 - nl);
   if (lo2 <= hi1) lo2 = hi1 + 1;
+  const int n_sink = hi1 + 1;
+  const int n_tiles = n_sink + max(0, mbl - lo2 + 1);
+  // The band is walked circularly, starting at the tile whose index is a multiple of the band
+  // length: step u visits the band tile congruent to u.  Work-groups of one head whose bands
+  // overlap (neighbouring query tiles, resident on the same XCD at the same time) then ask for
+  // the same K/V tile at the same step and share it in L2.  The order is free: online softmax
+  // does not care, liveness and the causal mask go by tile index.
+  const int n_band = n_tiles - n_sink;
+  const int band_rot = n_band > 0 ? (n_band - lo2 % n_band) % n_band : 0;
+  auto tile_at = [&](int t) __attribute__((always_inline)) {
+    if (t < n_sink) return t;
+    int u = t - n_sink + band_rot;
+    if (u >= n_band) u -= n_band;
+    return lo2 + u;
+  };
   // this wave's own live set
   const int w_hi1 = min(ns - 1, mbw);
   const int w_lo2 = max(0, mbw + 1 - nl);
+  auto live_tile = [&](int j) __attribute__((always_inline)) { return wave_has_rows && (j <= w_hi1 || (j >= w_lo2 && j <= mbw)); };
+  auto live = [&](int t) __attribute__((always_inline)) { return t >= 0 && t < n_tiles && live_tile(tile_at(t)); };
 
   const int64_t m_glob = (int64_t)qt * kQRows + wave * kWRows + mcol;   // this lane's query row
+
+  if (n_tiles == 0) {   // nothing is visible from this query tile: zeros
+    if (wave_has_rows && m_glob < N) {
+      uint16_t* orow = o + b * os.b + hq * os.h + m_glob * os.n;
+      u32x2 z = {0, 0};
+#pragma unroll
+      for (int i = 0; i < D / 8; ++i) *reinterpret_cast<u32x2*>(orow + 8 * i + 4 * g) = z;
+    }
+    return;
+  }
+
+  // ---- async tile copies: wave w, copy i fills chunks [(w*LPW+i)*64, +64) of a stage --------
+  const uint16_t* kbase = k + b * ks.b + hk * ks.h;   // uniform
+  const uint16_t* vbase = v + b * vs.b + hk * vs.h;
+  uint32_t koff[LPW], voff[LPW];
+#pragma unroll
+  for (int i = 0; i < LPW; ++i) {
+    const int L = (wave * LPW + i) * 64 + lane;     // chunk position inside the stage
+    const int row = L / CPR, pos = L % CPR;
+    koff[i] = 2u * ((uint32_t)(row * ks.n) + (uint32_t)((pos ^ ((row / RSH) % CPR)) * 8));   // bytes
+    voff[i] = 2u * ((uint32_t)(row * vs.n) + (uint32_t)((pos ^ (4 * ((row / RSH) % (CPR / 4)))) * 8));
+  }
+  // rows >= N of the ragged last tile repeat row N-1: their scores are masked, their softmax
+  // weight is exactly 0, and a repeated real row is finite
+  auto issue_tile = [&](const uint16_t* base, int64_t stride_n, const uint32_t (&off)[LPW], bool is_k,
+                        int j, char* stage) {
+    const uint16_t* src = base + (int64_t)j * kKV * stride_n;
+    const uint32_t dst = lds_address(stage) + wave * LPW * 1024;
+    if ((j + 1) * kKV <= N) {
+#pragma unroll
+      for (int i = 0; i < LPW; ++i) async_copy16(src, off[i], dst + i * 1024);
+    } else {
+      const int last = N - 1 - j * kKV;
+#pragma unroll
+      for (int i = 0; i < LPW; ++i) {
+        const int L = (wave * LPW + i) * 64 + lane;
+        const int row = L / CPR, pos = L % CPR;
+        const int sw = is_k ? ((row / RSH) % CPR) : (4 * ((row / RSH) % (CPR / 4)));
+        async_copy16(src, 2u * ((uint32_t)(min(row, last) * stride_n) + (uint32_t)((pos ^ sw) * 8)), dst + i * 1024);
+      }
+    }
+  };
+  auto issue_k = [&](int t) __attribute__((always_inline)) { issue_tile(kbase, ks.n, koff, true, tile_at(t), s_k + (t % kStages) * TILE_B); };
+  auto issue_v = [&](int t) __attribute__((always_inline)) { issue_tile(vbase, vs.n, voff, false, tile_at(t), s_v + (t % kStages) * TILE_B); };
+  auto batch_size = [&](int s) __attribute__((always_inline)) { return (s < 0) ? 0 : ((s + 3 < n_tiles) ? LPW : 0) + ((s + 2 < n_tiles) ? LPW : 0); };
+
+  // The matrix phase of iteration t reads K(t) and V(t-1) and starts the copies of K(t+3) and
+  // V(t+2), whose stages were last read in iteration t-1 by both groups.  Before the loop:
+  // K(0..2), V(0..1).
+  issue_k(0);
+  issue_v(0);
+  if (n_tiles > 1) { issue_k(1); issue_v(1); }
+  if (n_tiles > 2) issue_k(2);
 
   // ---- Q fragment (B operand): Q[m][16*ks + 8*g .. +7] ---------------------
   u32x4 qf[KS];
@@ -167,185 +324,188 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_kernel(
   for (int t = 0; t < DT; ++t)
 #pragma unroll
     for (int i = 0; i < 16; ++i) oacc[t][i] = 0.f;
+  f32x16 st[2];              // S^T of the current tile
+  uint32_t pf[16];           // P^T of the current tile, packed pairs, B-operand order
+#pragma unroll
+  for (int i = 0; i < 16; ++i) pf[i] = 0;
   float m_run = -INFINITY;   // reference max of scale_log2 * s used by exp2 (lags the true max by <= kRescaleStep)
   float l_run = 0.f;         // this lane's share of the running sum (the lane+32 twin holds the rest)
 
-  // ---- cooperative tile load: thread -> (row, 16-byte chunk) ----------------
-  const int ld_row = tid / CPR;
-  const int ld_chk = tid % CPR;
-  const uint16_t* kbase = k + b * ks.b + hk * ks.h;   // uniform
-  const uint16_t* vbase = v + b * vs.b + hk * vs.h;
-  uint32_t koff[PASSES], voff[PASSES];                // element offsets inside a tile
+  // ---- operand read addresses: LDS byte address of stage 0, row 0 of this lane; stage, half and
+  // k-step go into the instruction's immediate offset, so the matrix phase needs no VALU work ----
+  uint32_t k_ad[KS];
+  {
+    const uint32_t k_rd = (uint32_t)(mcol * ROW_B) | (uint32_t)(((g ^ ((mcol / RSH) % CPR)) & (CPR - 1)) * 16);
 #pragma unroll
-  for (int p = 0; p < PASSES; ++p) {
-    koff[p] = (uint32_t)((p * RPP + ld_row) * ks.n + ld_chk * 8);
-    voff[p] = (uint32_t)((p * RPP + ld_row) * vs.n + ld_chk * 8);
+    for (int s = 0; s < KS; ++s) k_ad[s] = lds_address(s_k) + (k_rd ^ (uint32_t)(32 * s));
   }
-  u32x4 kreg[PASSES], vreg[PASSES];
+  uint32_t v_ad[DT];
+  {
+    const int grp16 = lane & 15;
+    const int dhalf = (lane >> 4) & 1;
+    const int v_row = 4 * g + (grp16 >> 2);
+    const uint32_t v_rd = (uint32_t)(v_row * ROW_B) +
+                          (uint32_t)(((2 * dhalf + ((grp16 & 3) >> 1)) ^ (4 * ((v_row / RSH) % (CPR / 4)))) * 16 +
+                                     8 * (grp16 & 1));
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) v_ad[dt] = lds_address(s_v) + (v_rd ^ (uint32_t)(64 * dt));
+  }
 
-  auto issue_loads = [&](int j) {
-    const uint16_t* kt = kbase + (int64_t)j * kKV * ks.n;
-    const uint16_t* vt = vbase + (int64_t)j * kKV * vs.n;
-    if ((j + 1) * kKV <= N) {
-#pragma unroll
-      for (int p = 0; p < PASSES; ++p) {
-        kreg[p] = *reinterpret_cast<const u32x4*>(kt + koff[p]);
-        vreg[p] = *reinterpret_cast<const u32x4*>(vt + voff[p]);
+  // Matrix phase of one iteration: P.V of the previous tile and Q.K^T of the current one,
+  // alternating, operands fetched kAhead MFMAs ahead.  k_ad / v_ad point at the stages to read.
+  // Slot i: even -> P.V op i/2 (k-step (i/2)/DT, d tile (i/2)%DT), odd -> Q.K^T op i/2
+  // (half (i/2)%2, k-step (i/2)/2).
+  auto matrix_phase = [&]() __attribute__((always_inline)) {
+    constexpr int kSlots = 4 * DT + 2 * KS;
+    constexpr int kAhead = 6;
+    u32x4 opnd[kSlots];
+    auto fetch = [&](int i) __attribute__((always_inline)) {
+      const int j = i >> 1;
+      if (i & 1) {
+        opnd[i] = lds_load16(k_ad[j >> 1], (j & 1) * 32 * ROW_B);
+      } else {
+        const int tk = j / DT, dt = j % DT;
+        const u32x2 lo = lds_load_tr16(v_ad[dt], (16 * tk) * ROW_B);
+        const u32x2 hi = lds_load_tr16(v_ad[dt], (16 * tk + 8) * ROW_B);
+        opnd[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
       }
-    } else {   // the ragged last tile: rows >= N read as zero
+    };
+    auto op = [&](int i) __attribute__((always_inline)) {
+      const int j = i >> 1;
+      if (i & 1) {
+        const int nt = j & 1, s = j >> 1;
+        if (s == 0) {
+          f32x16 z;
 #pragma unroll
-      for (int p = 0; p < PASSES; ++p) {
-        const bool ok = j * kKV + p * RPP + ld_row < N;
-        u32x4 z = {0, 0, 0, 0};
-        kreg[p] = ok ? *reinterpret_cast<const u32x4*>(kt + koff[p]) : z;
-        vreg[p] = ok ? *reinterpret_cast<const u32x4*>(vt + voff[p]) : z;
+          for (int e = 0; e < 16; ++e) z[e] = 0.f;
+          st[nt] = T::mfma(opnd[i], qf[0], z);
+        } else {
+          st[nt] = T::mfma(opnd[i], qf[s], st[nt]);
+        }
+      } else {
+        const int tk = j / DT, dt = j % DT;
+        const u32x4 bfrag = {pf[4 * tk], pf[4 * tk + 1], pf[4 * tk + 2], pf[4 * tk + 3]};
+        oacc[dt] = T::mfma(opnd[i], bfrag, oacc[dt]);
       }
+    };
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) fetch(i);
+#pragma unroll
+    for (int i = 0; i < kSlots; ++i) {
+      if (i + kAhead < kSlots) fetch(i + kAhead);
+      op(i);
+      __builtin_amdgcn_sched_barrier(0);   // keeps the operand reads kAhead MFMAs ahead of their use
     }
   };
-  auto store_tile = [&](int buf) {
+  // Q.K^T only (the first iteration)
+  auto qk_phase = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const int r = p * RPP + ld_row;
-      *reinterpret_cast<u32x4*>(s_k + buf * KTILE + r * LDK + ld_chk * 8) = kreg[p];
-      *reinterpret_cast<u32x4*>(s_v + buf * VTILE + r * LDV + ld_chk * 8) = vreg[p];
+    for (int nt = 0; nt < 2; ++nt) {
+      u32x4 kf[KS];
+#pragma unroll
+      for (int s = 0; s < KS; ++s) kf[s] = lds_load16(k_ad[s], nt * 32 * ROW_B);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) st[nt][i] = 0.f;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) st[nt] = T::mfma(kf[s], qf[s], st[nt]);
     }
   };
-  auto next_tile = [&](int j) { return (j == hi1) ? lo2 : j + 1; };
-
-  // operand read positions inside a buffer
-  const int k_rd_off = mcol * LDK + 8 * g;                               // + 32*nt*LDK + 16*ks
-  const int grp16 = lane & 15;
-  const int dhalf = (lane >> 4) & 1;
-  const int v_rd_off = (4 * g + (grp16 >> 2)) * LDV + 16 * dhalf + 4 * (grp16 & 3);
-                                                                         // + (16*t [+8])*LDV + 32*dt
-
-  int j = (hi1 >= 0) ? 0 : lo2;
-  if (j > mb1) {   // nothing is visible from this query tile: zeros
-    if (wave_has_rows && m_glob < N) {
-      uint16_t* orow = o + b * os.b + hq * os.h + m_glob * os.n;
-      u32x2 z = {0, 0};
-#pragma unroll
-      for (int i = 0; i < D / 8; ++i) *reinterpret_cast<u32x2*>(orow + 8 * i + 4 * g) = z;
-    }
-    return;
-  }
-  issue_loads(j);
-  store_tile(0);
-  int jn = next_tile(j);
-  if (jn <= mb1) issue_loads(jn);
-  __syncthreads();
-
-  int buf = 0;
-  while (true) {
-    const bool live = wave_has_rows && (j <= w_hi1 || (j >= w_lo2 && j <= mbw));
-    if (live) {
-      const uint16_t* k_rd = s_k + buf * KTILE + k_rd_off;
-      const uint16_t* v_rd = s_v + buf * VTILE + v_rd_off;
-      // ---- S^T = K Q^T : two 32-key tiles; the operand reads run kPre MFMAs ahead ----
-      f32x16 st[2];
-      {
-        constexpr int kPre = 8;
-        u32x4 a[2 * KS];
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-          for (int s = 0; s < KS; ++s)
-            a[nt * KS + s] = *reinterpret_cast<const u32x4*>(k_rd + nt * 32 * LDK + 16 * s);
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-#pragma unroll
-          for (int i = 0; i < 16; ++i) st[nt][i] = 0.f;
-#pragma unroll
-          for (int s = 0; s < KS; ++s) st[nt] = T::mfma(a[nt * KS + s], qf[s], st[nt]);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x100, kPre < 2 * KS ? kPre : 2 * KS, 0);
-#pragma unroll
-        for (int i = 0; i < 2 * KS - kPre; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, kPre < 2 * KS ? kPre : 2 * KS, 0);
-      }
-      // ---- causal mask on the diagonal tile ----
-      if (j == mbw) {
-        const int m_in = (wave & 1) * kWRows + mcol;   // row inside the 64-row block
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int n_in = nt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-            if (n_in > m_in) st[nt][i] = -INFINITY;
-          }
-      }
-      // ---- online softmax, base 2, with a lagging reference max ----
-      float mx = st[0][0];
+  // mask + online softmax of tile j: st -> pf, updates m_run, l_run (and rescales oacc when needed;
+  // every P.V issued so far belongs to earlier tiles and has completed in this wave's matrix phase)
+  auto softmax = [&](int j) __attribute__((always_inline)) {
+    if (j == mbw) {   // causal mask on the diagonal tile
+      const int m_in = (wave & 1) * kWRows + mcol;   // row inside the 64-row block
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, st[nt][i]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_cand = mx * scale_log2;   // finite: a live tile has a visible key in every row
-      // exp2 arguments stay <= kRescaleStep as long as no row max outgrew its reference by more
-      // than that; only then are O and l rescaled (a wave-uniform, rare branch after the first tile)
-      if (__any(m_cand > m_run + kRescaleStep)) {
-        const float m_new = fmaxf(m_run, m_cand);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        l_run *= alpha;
+        for (int i = 0; i < 16; ++i) {
+          const int n_in = nt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+          if (n_in > m_in) st[nt][i] = -INFINITY;
+        }
+    }
+    float mx = st[0][0];
 #pragma unroll
-        for (int t = 0; t < DT; ++t)
+    for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) oacc[t][i] *= alpha;
-        m_run = m_new;
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, st[nt][i]);
+    mx = max_with_other_half(mx);
+    const float m_cand = mx * scale_log2;   // finite: a live tile has a visible key in every row
+    if (__any(m_cand > m_run + kRescaleStep)) {
+      const float m_new = fmaxf(m_run, m_cand);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      l_run *= alpha;
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[t][i] *= alpha;
+      m_run = m_new;
+    }
+    float psum[2] = {0.f, 0.f};   // two chains: a dot2 result is not ready for the very next instruction
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i], scale_log2, -m_run));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i + 1], scale_log2, -m_run));
+        const uint32_t pk = T::pack(p0, p1);
+        pf[nt * 8 + (i >> 1)] = pk;
+        psum[(i >> 1) & 1] = T::add_pair(pk, psum[(i >> 1) & 1]);   // the sum of what P.V multiplies with: the rounded weights
       }
-      float psum = 0.f;
-      uint32_t pf[16];
+    l_run += psum[0] + psum[1];
+  };
+
+  wait_vm(0);
+  // the Q loads have landed too; pin that fact here so that the compiler does not put its own
+  // vmcnt(0) wait at their first use inside the loop, where it would also wait for the copies
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
+  for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[s]));
+  phase_barrier();               // K(0..2) and V(0..1) are in LDS
+
+  // Iteration t: matrix phase = P.V of tile t-1 and Q.K^T of tile t, then softmax phase = tile t.
+  // There is one work-group barrier per iteration; group A meets it after its softmax phase, group
+  // B after its matrix phase, so B's softmax of tile t runs beside A's matrix phase of tile t+1 and
+  // each SIMD holds one wave in either phase.  A wave for which tile t-1 or t is not live still
+  // runs the whole matrix phase (with P = 0, or ignoring S), which keeps the loop body a single
+  // straight block; it skips the phase when neither is live.  The copies started in iteration t
+  // overwrite the stages of K(t-1) and V(t-2), which every wave has finished reading before
+  // barrier t-1; the copies started two iterations ago (K(t+1), V(t)) are first read after barrier
+  // t, and every wave waits for its own before it.  Iteration n_tiles only finishes P.V of the
+  // last tile.
+  auto iteration = [&](int t, auto FIRST) __attribute__((always_inline)) {
+    constexpr bool kFirst = decltype(FIRST)::value != 0;
+    const int n_wait = batch_size(t - 1) + batch_size(t);
+    // ---------------- matrix phase ----------------
+    if (t + 3 < n_tiles) issue_k(t + 3);
+    if (t + 2 < n_tiles) issue_v(t + 2);
+    const bool lp = live(t - 1), lc = live(t);
+    if (kFirst) {
+      if (lc) qk_phase();
+    } else {
+      if (lp || lc) matrix_phase();
+    }
+    if (grp == 1) { wait_vm(n_wait); phase_barrier(); }
+    // ---------------- softmax phase ----------------
+    if (lc) {
+      softmax(tile_at(t));
+    } else if (lp) {   // the next matrix phase this wave runs must add nothing for a dead tile
 #pragma unroll
-        for (int i = 0; i < 16; i += 2) {
-          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i], scale_log2, -m_run));
-          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i + 1], scale_log2, -m_run));
-          psum += p0 + p1;
-          pf[nt * 8 + (i >> 1)] = T::pack(p0, p1);
-        }
-      l_run += psum;
-      // ---- O^T += V^T P^T ; operand reads run kPre MFMAs ahead ----
-      {
-        constexpr int kPre = 4;
-        u32x4 a[4 * DT];
+      for (int i = 0; i < 16; ++i) pf[i] = 0;
+    }
+    // advance the operand addresses to the next stages (K: t+1, V: t)
+    {
+      const int kd = ((t + 1) % kStages == 0) ? -(kStages - 1) * TILE_B : TILE_B;
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+      for (int s = 0; s < KS; ++s) k_ad[s] += kd;
+      if (!kFirst) {
+        const int vd = (t % kStages == 0) ? -(kStages - 1) * TILE_B : TILE_B;
 #pragma unroll
-          for (int dt = 0; dt < DT; ++dt) {
-            const u32x2 lo = lds_read_tr16(v_rd + (16 * t) * LDV + 32 * dt);
-            const u32x2 hi = lds_read_tr16(v_rd + (16 * t + 8) * LDV + 32 * dt);
-            a[t * DT + dt] = u32x4{lo.x, lo.y, hi.x, hi.y};
-          }
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const u32x4 bfrag = {pf[4 * t], pf[4 * t + 1], pf[4 * t + 2], pf[4 * t + 3]};
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) oacc[dt] = T::mfma(a[t * DT + dt], bfrag, oacc[dt]);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 * kPre, 0);
-#pragma unroll
-        for (int i = 0; i < 4 * DT - kPre; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, kPre, 0);
+        for (int dt = 0; dt < DT; ++dt) v_ad[dt] += vd;
       }
     }
-    if (jn > mb1) break;
-    // tile jn (in registers since the previous iteration) goes into the other buffer; every wave
-    // left that buffer before the last barrier
-    store_tile(buf ^ 1);
-    j = jn;
-    jn = next_tile(j);
-    if (jn <= mb1) issue_loads(jn);
-    __syncthreads();
-    buf ^= 1;
-  }
+    if (grp == 0) { wait_vm(n_wait); phase_barrier(); }
+  };
+  iteration(0, IC<1>{});   // no P.V yet (and no V stage to read)
+  for (int t = 1; t <= n_tiles; ++t) iteration(t, IC<0>{});
 
   // ---- epilogue: O[m][d] = O^T[d][m] / l ---------------------------------
   if (!wave_has_rows || m_glob >= N) return;
@@ -366,7 +526,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_kernel(
 
 template <typename T, int D>
 static size_t prefill_lds_bytes() {
-  return (size_t)2 * kKV * ((D + 8) + (D + 32)) * sizeof(uint16_t);
+  return (size_t)2 * kStages * kKV * D * sizeof(uint16_t);   // K stages + V stages
 }
 
 template <typename T, int D>
@@ -378,6 +538,9 @@ static int launch_prefill(const void* q, const void* k, const void* v, void* o, 
   const int BH = B * Hq;
   const int64_t groups = (int64_t)((BH + 7) / 8) * 8 * n_qtiles;
   if (groups > 0x7fffffffLL) return fail(MOA_ERR_UNSUPPORTED, "moa_prefill_fwd: too many work-groups");
+  // the async copies address a tile row through a 32-bit element offset
+  if (64 * ks[2] + D >= (1ll << 31) || 64 * vs[2] + D >= (1ll << 31))
+    return fail(MOA_ERR_UNSUPPORTED, "moa_prefill_fwd: k/v token stride too large");
   Strides4 sq = {qs[0], qs[1], qs[2]}, sk = {ks[0], ks[1], ks[2]}, sv = {vs[0], vs[1], vs[2]},
            so = {os[0], os[1], os[2]};
   const size_t lds = prefill_lds_bytes<T, D>();
@@ -410,6 +573,7 @@ static int check_strides(const char* name, const int64_t* s, const void* p) {
 }  // namespace moa
 
 using namespace moa;
+
 
 extern "C" int moa_prefill_fwd(const void* q, const void* k, const void* v, void* o,
                                const int64_t* q_strides, const int64_t* k_strides,
