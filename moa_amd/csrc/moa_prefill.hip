@@ -59,6 +59,7 @@ constexpr int kQRows = 256;   // query rows per work-group
 constexpr int kWRows = 32;    // query rows per wave
 constexpr int kKV = 64;       // keys per tile (the sparsity block)
 constexpr int kStages = 4;    // LDS stages per tensor
+constexpr int kMaxSortedHeads = 1024;   // kv heads the span-sorted schedule handles (else: given order)
 constexpr float kLog2eF = 1.4426950408889634f;
 
 struct PF16 {
@@ -198,28 +199,47 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
   char* const s_v = s_mem + kStages * TILE_B;
 
   // ---- which (head, query tile) --------------------------------------------
-  // Work-groups are dealt to the 8 XCDs round-robin by the hardware.  Group
-  // idx goes to XCD idx%8 and is the (idx/8)-th one there; an XCD owns the heads
-  // congruent to it mod 8 and walks them one after the other, late (long) query
-  // tiles first, so that the groups resident on an XCD share one head's K/V in L2.
+  // Work-groups are dealt to the 8 XCDs round-robin by the hardware: group idx goes to XCD idx%8
+  // and is the (idx/8)-th one there.  An XCD walks (batch, head) pairs one after the other, late
+  // (long) query tiles first, so that the groups resident on it share one head's K/V in L2.
+  // Heads differ a lot in span, so the pairs are dealt to the XCDs from a list sorted by
+  // decreasing span, in snake order (0..7, 7..0, ...): every XCD gets about the same work and
+  // takes its long heads first, its short ones last.
+  const int tid = threadIdx.x;
+  const int Hkv = Hq / group;
+  const int nb = (N + kKV - 1) / kKV;
+  __shared__ int s_head_of_rank[kMaxSortedHeads];
+  const bool sorted = Hkv <= kMaxSortedHeads;
+  if (sorted) {
+    for (int h = tid; h < Hkv; h += kPfThreads) {
+      const int64_t wh = min((int64_t)nb, sink_blocks[h] + local_blocks[h]);
+      int rank = 0;
+      for (int j = 0; j < Hkv; ++j) {
+        const int64_t wj = min((int64_t)nb, sink_blocks[j] + local_blocks[j]);
+        rank += (wj > wh) || (wj == wh && j < h);
+      }
+      s_head_of_rank[rank] = h;
+    }
+    __syncthreads();
+  }
   const int xcd = blockIdx.x & 7;
   const int seq = blockIdx.x >> 3;
-  const int heads_here = (BH - xcd + 7) >> 3;
-  if (seq >= heads_here * n_qtiles) return;
-  const int bh = (seq / n_qtiles) * 8 + xcd;
+  const int round = seq / n_qtiles;                                // this XCD's round-th pair
+  const int pos = round * 8 + ((round & 1) ? 7 - xcd : xcd);      // position in the sorted list
+  if (pos >= BH) return;
+  // sorted list: kv heads by rank; per kv head, batch-major, then the query heads of its group
+  const int per_head = (BH / Hq) * group;
+  const int hk = __builtin_amdgcn_readfirstlane(sorted ? s_head_of_rank[pos / per_head] : pos / per_head);
+  const int b = (pos % per_head) / group;
+  const int hq = hk * group + pos % group;
   const int qt = n_qtiles - 1 - (seq % n_qtiles);
-  const int b = bh / Hq;
-  const int hq = bh % Hq;
-  const int hk = hq / group;
 
-  const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int grp = wave >> 2;    // 0: group A, 1: group B (one phase behind A)
   const int mcol = lane & 31;   // query row inside the wave's 32 (the MFMA column)
   const int g = lane >> 5;      // half-wave
 
-  const int nb = (N + kKV - 1) / kKV;
   const int ns = __builtin_amdgcn_readfirstlane((int)sink_blocks[hk]);
   const int nl = __builtin_amdgcn_readfirstlane((int)local_blocks[hk]);
   const int mb0 = 4 * qt;                                  // first query block of the group
