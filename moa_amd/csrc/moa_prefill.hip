@@ -59,7 +59,7 @@ constexpr int kQRows = 256;   // query rows per work-group
 constexpr int kWRows = 32;    // query rows per wave
 constexpr int kKV = 64;       // keys per tile (the sparsity block)
 constexpr int kStages = 4;    // LDS stages per tensor
-constexpr int kMaxSortedHeads = 1024;   // kv heads the span-sorted schedule handles (else: given order)
+constexpr int kMaxSortedHeads = 512;   // kv heads the span-sorted schedule handles (else: given order)
 constexpr float kLog2eF = 1.4426950408889634f;
 
 struct PF16 {
@@ -208,14 +208,21 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
   const int tid = threadIdx.x;
   const int Hkv = Hq / group;
   const int nb = (N + kKV - 1) / kKV;
-  __shared__ int s_head_of_rank[kMaxSortedHeads];
+  __shared__ int s_head_of_rank[kMaxSortedHeads], s_ns[kMaxSortedHeads], s_nl[kMaxSortedHeads];
   const bool sorted = Hkv <= kMaxSortedHeads;
+  // block counts clamped to [0, nb]: beyond that range they select the same tiles
+  auto clamp_blocks = [&](int64_t x) __attribute__((always_inline)) { return (int)max((int64_t)0, min((int64_t)nb, x)); };
   if (sorted) {
     for (int h = tid; h < Hkv; h += kPfThreads) {
-      const int64_t wh = min((int64_t)nb, sink_blocks[h] + local_blocks[h]);
+      s_ns[h] = clamp_blocks(sink_blocks[h]);
+      s_nl[h] = clamp_blocks(local_blocks[h]);
+    }
+    __syncthreads();
+    for (int h = tid; h < Hkv; h += kPfThreads) {
+      const int wh = min(nb, s_ns[h] + s_nl[h]);
       int rank = 0;
       for (int j = 0; j < Hkv; ++j) {
-        const int64_t wj = min((int64_t)nb, sink_blocks[j] + local_blocks[j]);
+        const int wj = min(nb, s_ns[j] + s_nl[j]);
         rank += (wj > wh) || (wj == wh && j < h);
       }
       s_head_of_rank[rank] = h;
@@ -240,8 +247,8 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
   const int mcol = lane & 31;   // query row inside the wave's 32 (the MFMA column)
   const int g = lane >> 5;      // half-wave
 
-  const int ns = __builtin_amdgcn_readfirstlane((int)sink_blocks[hk]);
-  const int nl = __builtin_amdgcn_readfirstlane((int)local_blocks[hk]);
+  const int ns = __builtin_amdgcn_readfirstlane(sorted ? s_ns[hk] : clamp_blocks(sink_blocks[hk]));
+  const int nl = __builtin_amdgcn_readfirstlane(sorted ? s_nl[hk] : clamp_blocks(local_blocks[hk]));
   const int mb0 = 4 * qt;                                  // first query block of the group
   const int mbl = min(4 * qt + 3, nb - 1);                 // last one that exists
   const int mbw = 4 * qt + (wave >> 1);                    // this wave's query block
