@@ -156,6 +156,46 @@ def bench_decode(torch, dev, args):
     }
 
 
+def bench_rope_append(torch, dev, args, cache, iters=50):
+    """The step in front of the decode kernel at the headline shape: rotary embedding of q and k
+    plus the ring append, as ONE launch (StaticCircularCache.rope_update) and as the two launches
+    it replaces (rotary kernel, then append)."""
+    from moa_amd.kernels.rotary import apply_rotary_pos_emb
+    from moa_amd.workloads import rope_append_bytes
+
+    B, H, D = args.batch, 32, 128
+    dtype = torch.float16
+    gen = torch.Generator(device=dev).manual_seed(5)
+    q, k, v = (torch.randn(B, 1, H, D, generator=gen, device=dev, dtype=dtype).transpose(1, 2) for _ in range(3))
+    ang = torch.rand(B, 1, D, generator=gen, device=dev) * 6.28
+    cos, sin = ang.cos().to(dtype), ang.sin().to(dtype)
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize(dev)
+        evs = []
+        for _ in range(iters):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            evs.append((e0, e1))
+        torch.cuda.synchronize(dev)
+        ms = sorted(a.elapsed_time(b) for a, b in evs)
+        return ms[len(ms) // 2] * 1e3
+
+    def separate():
+        qe, ke = apply_rotary_pos_emb(q, k, cos, sin)
+        cache.update(ke, v, 0)
+
+    fused_us = timed(lambda: cache.rope_update(q, k, v, cos, sin, 0))
+    separate_us = timed(separate)
+    nbytes = rope_append_bytes(B, H, D)
+    return {"fused_us": fused_us, "separate_us": separate_us, "bytes": nbytes,
+            "GB/s": nbytes / (fused_us * 1e-6) / 1e9}
+
+
 def bench_prefill(torch, dev, args):
     from moa_amd import mixture_of_sparse_attention
     from moa_amd.workloads import elastic_spans, prefill_work
@@ -268,6 +308,7 @@ def main():
         print(json.dumps({"prefill": bench_prefill(torch, dev, args)}))
         return
     dec = bench_decode(torch, dev, args)
+    rope = bench_rope_append(torch, dev, args, dec["cache"])
     del dec["cache"]
     if args.only == "decode":
         print(json.dumps({"decode": dec}))
@@ -317,6 +358,7 @@ def main():
         },
         "cpu_baseline": cpu,
         "append": {"us": dec["append_us"], "bytes": dec["append_bytes"], "GB/s": dec["append_gbs"]},
+        "rope_append": rope,
         "prefill": pre,
     }
     print(json.dumps(line))

@@ -124,6 +124,48 @@ int moa_cache_append(const void* k_new, const void* v_new,
                      int64_t kv_len, int B, int H, int D, int64_t sumC,
                      int dtype, void* stream);
 
+/*
+ * Rotary position embedding of the query and key heads (prompt or single step).
+ * Replaces: apply_rotary_pos_emb(query_states, key_states, cos, sin) in the
+ * reference's caller (MoA/models/llama/modeling_llama.py:252; the function is
+ * transformers 4.44.2's, requirements.txt:8):
+ *   x_embed = (x * cos) + (rotate_half(x) * sin),  rotate_half(x) = cat(-x[D/2:], x[:D/2]),
+ * rounded to the tensors' dtype after each product and after the sum, as torch
+ * evaluates it (results are bit-identical to that evaluation).
+ * q, k, q_out, k_out: [B, H, N, D] through host strides (4 element strides,
+ * order B,H,N,D; D stride 1); q_out == q and k_out == k (in place) is allowed.
+ * cos, sin: [B, N, D] through cs_strides (3 element strides; a batch stride of 0
+ * broadcasts one position table).  Hq or Hkv may be 0 to rotate one tensor only.
+ * head_dim * element size must be a multiple of 32 bytes.  f16, bf16, f32.
+ */
+int moa_rope_fwd(const void* q, const void* k, void* q_out, void* k_out,
+                 const int64_t* q_strides, const int64_t* k_strides,
+                 const int64_t* qo_strides, const int64_t* ko_strides,
+                 const void* cos, const void* sin, const int64_t* cs_strides,
+                 int B, int Hq, int Hkv, int N, int D, int dtype, void* stream);
+
+/*
+ * One decode step in front of the attention kernel, in one launch: rotary
+ * embedding of q (written to q_out, contiguous [B, Hq, D] = the reference's
+ * [B,1,Hq,D]) and of k, and the append of the rotated k and of v into every
+ * head's ring with the index bookkeeping of moa_cache_append.
+ * Replaces: modeling_llama.py:252 (apply_rotary_pos_emb) + :262
+ * (past_key_value.update, decode branch cache_utils.py:1020-1058).
+ * q_new, k_new, v_new: [B, H, D] through host strides (3 element strides,
+ * order B,H,D; D stride 1); cos, sin: [B, D] rows cs_stride_b elements apart
+ * (0 broadcasts).  The other arguments are those of moa_cache_append; kc and vc
+ * are required.
+ */
+int moa_rope_cache_append(const void* q_new, const void* k_new, const void* v_new,
+                          const int64_t* qn_strides, const int64_t* kn_strides,
+                          const int64_t* vn_strides, const void* cos, const void* sin,
+                          int64_t cs_stride_b, void* q_out, void* kc, void* vc,
+                          int64_t* mask_cache, int64_t* update_index, int64_t* valid_len,
+                          const int64_t* circ_head, const int64_t* circ_size,
+                          const int64_t* static_size, const int64_t* max_len,
+                          int64_t kv_len, int B, int Hq, int Hkv, int D, int64_t sumC,
+                          int dtype, void* stream);
+
 /* Scratch bytes for moa_cache_prefill_insert when an attention_mask is given
  * (0 otherwise). */
 size_t moa_cache_prefill_workspace_bytes(int B, int S);

@@ -44,6 +44,12 @@ SIGNATURES = {
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                          c_void_p, c_size_t, c_int64, c_int, c_int, c_int, c_int, c_int64,
                                          c_int64, c_int, c_void_p]),
+    "moa_rope_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, _I64P, _I64P, _I64P, _I64P, c_void_p,
+                             c_void_p, _I64P, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "moa_rope_cache_append": (c_int, [c_void_p, c_void_p, c_void_p, _I64P, _I64P, _I64P, c_void_p, c_void_p,
+                                      c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int,
+                                      c_int, c_int64, c_int, c_void_p]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

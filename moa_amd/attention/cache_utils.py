@@ -154,6 +154,71 @@ class StaticCircularCache:
             self.key_cache[layer_idx] = torch.zeros(shape, dtype=self.dtype, device=device)
             self.value_cache[layer_idx] = torch.zeros(shape, dtype=self.dtype, device=device)
 
+    def rope_update(
+        self,
+        query_states: Tensor,
+        key_states: Tensor,
+        value_states: Tensor,
+        cos: Tensor,
+        sin: Tensor,
+        layer_idx: int,
+        attention_mask: Optional[torch.IntTensor] = None,
+    ) -> Tuple[Tensor, Tensor, Tensor]:
+        """Rotary embedding of q and k followed by ``update``: the two steps the reference's caller
+        runs between the projections and the attention call (modeling_llama.py:252 and :262).
+
+        q ``[batch, q_heads, seq_len, head_dim]``, k/v ``[batch, heads, seq_len, head_dim]`` before
+        rotation, cos/sin ``[batch or 1, seq_len, head_dim]``.  Returns ``(q_embed, keys, values)``
+        where keys/values are what ``update`` returns.  With ``seq_len == 1`` this is ONE launch:
+        q is rotated into a ``[batch, 1, q_heads, head_dim]`` buffer (returned as its
+        ``[batch, q_heads, 1, head_dim]`` view, the layout the decode kernel takes without a copy), k is
+        rotated straight into its ring slot, v is copied into its slot.
+        """
+        from ..kernels.rotary import apply_rotary_pos_emb, _cos_sin_strides
+
+        seq_len = key_states.shape[-2]
+        if seq_len != 1 or not self.update_cache_content:
+            q_embed, k_embed = apply_rotary_pos_emb(query_states, key_states, cos, sin)
+            keys, values = self.update(k_embed, value_states, layer_idx, attention_mask)
+            return q_embed, keys, values
+
+        assert layer_idx < self.num_layers
+        H = self.num_head_for_each_layer[layer_idx]
+        device = key_states.device
+        if torch.device(device).type != "cuda":
+            raise _lib.MoaKernelError(
+                "StaticCircularCache.rope_update: tensors must live on the GPU; moa_amd has no CPU path")
+        B, Hq, _, D = query_states.shape
+        assert key_states.shape == (B, H, 1, D) and value_states.shape == key_states.shape
+        assert B == self.batch_size and D == self.head_dim
+        assert query_states.dtype == self.dtype and key_states.dtype == self.dtype and value_states.dtype == self.dtype
+        assert cos.dtype == self.dtype and sin.dtype == self.dtype, "cos/sin must have the cache dtype"
+        lib = _lib.load()
+        self._to_device(layer_idx, device)
+        if layer_idx == 0:
+            self.cache_position += 1
+        cos, sin, css = _cos_sin_strides(cos, sin, B, 1, D)
+        qn, kn, vn = (t[:, :, -1, :] for t in (query_states, key_states, value_states))
+        qn, kn, vn = (t if t.stride(-1) == 1 else t.contiguous() for t in (qn, kn, vn))
+        q_out = torch.empty((B, 1, Hq, D), dtype=self.dtype, device=device)
+        upd = self.cache_update_index[layer_idx]
+        assert upd.is_contiguous() and self.cache_valid_length[layer_idx].is_contiguous()
+        rc = lib.moa_rope_cache_append(
+            qn.data_ptr(), kn.data_ptr(), vn.data_ptr(), _lib.i64_array(qn.stride()), _lib.i64_array(kn.stride()),
+            _lib.i64_array(vn.stride()), cos.data_ptr(), sin.data_ptr(), css[0], q_out.data_ptr(),
+            self.key_cache[layer_idx].data_ptr(), self.value_cache[layer_idx].data_ptr(),
+            self.mask_cache[layer_idx].data_ptr(), upd.data_ptr(),
+            self.cache_valid_length[layer_idx].data_ptr(),
+            self.circular_cache_head_index[layer_idx].data_ptr(),
+            self.circular_cache_size[layer_idx].data_ptr(),
+            self.static_cache_size[layer_idx].data_ptr(),
+            self.cache_max_length[layer_idx].data_ptr(),
+            self._kv_len[layer_idx], B, Hq, H, D, self.layer_cache_size[layer_idx],
+            _lib.dtype_code(self.dtype), _lib.current_stream_ptr(device))
+        _lib.check(rc)
+        self._kv_len[layer_idx] += 1
+        return q_out.transpose(1, 2), self.key_cache[layer_idx], self.value_cache[layer_idx]
+
     def update(
         self,
         key_states: Tensor,

@@ -18,7 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "csrc", "build")
 LIB_PATH = os.path.join(HERE, "libmoa_hip.so")
 
-SOURCES = ["moa_capi.hip", "moa_cache.hip", "moa_decode.hip", "moa_prefill.hip"]
+SOURCES = ["moa_capi.hip", "moa_cache.hip", "moa_decode.hip", "moa_prefill.hip", "moa_rope.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -33,6 +33,10 @@ HIPCC_FLAGS = [
     # packed-FP32 instructions are switched off for all device code of this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+
+
+# moa_rope.hip reproduces torch's per-operation rounding bit for bit: no multiply-add contraction there
+PER_SOURCE_FLAGS = {"moa_rope.hip": ["-ffp-contract=off"]}
 
 
 def _hipcc() -> str:
@@ -55,7 +59,7 @@ def is_stale() -> bool:
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
     extra = os.environ.get("MOA_HIPCC_FLAGS", "").split()   # e.g. -DNAME for an experiment build
-    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *PER_SOURCE_FLAGS.get(src, []), *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")

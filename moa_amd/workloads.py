@@ -76,6 +76,12 @@ def decode_bytes(valid_rows_total: int, batch: int, heads: int, head_dim: int, e
     return valid_rows_total * head_dim * 2 * elem + 2 * batch * heads * head_dim * elem + 16 * batch * heads
 
 
+def rope_append_bytes(batch: int, heads: int, head_dim: int, elem: int = 2) -> int:
+    """fused rotary + append step: q, k, v read, q and two cache rows written, cos and sin read,
+    plus the append's index traffic."""
+    return (6 * batch * heads * head_dim + 2 * batch * head_dim) * elem + 40 * batch * heads
+
+
 def append_bytes(batch: int, heads: int, head_dim: int, elem: int = 2) -> int:
     """new k, v read + two rows written + update_index r/w, valid_len r/w, mask write."""
     return 4 * batch * heads * head_dim * elem + 40 * batch * heads

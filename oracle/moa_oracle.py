@@ -30,6 +30,11 @@ reference checkout).  What pins each function (see tests/test_oracle_*.py):
       both are checked against golden vectors in tests/golden/.
   moa_config_to_cache_config        hand-computed known answers + shipped
       plans.
+  rope_reference                    the published formula of transformers'
+      apply_rotary_pos_emb (the reference's pinned dependency, not vendored);
+      checked bit for bit against the installed transformers' function, a
+      hand-computed known answer, identity at position 0, norm preservation
+      and the relative-position property in fp64.
 
 Parity unpinned (no reference test, fixture or runnable implementation covers
 it): the external ``flashinfer.moa_decode`` CUDA op.  Its semantics are taken
@@ -499,3 +504,43 @@ def moa_config_to_cache_config(moa_config: dict, seq_len: int, max_new_token: in
         cache.append(cl)
         static.append(sl)
     return {"cache_size": cache, "static_size": static}
+
+
+# --------------------------------------------------------------------------
+# Rotary position embedding (the step in front of the path)
+# --------------------------------------------------------------------------
+
+
+def rope_reference(x, cos, sin):
+    """``x*cos + rotate_half(x)*sin`` evaluated by torch on the CPU in x's dtype.
+
+    Restates transformers 4.44.2 ``apply_rotary_pos_emb`` / ``rotate_half``
+    (models/llama/modeling_llama.py of that package; the reference pins it in
+    requirements.txt:8 and calls it at MoA/models/llama/modeling_llama.py:252).
+    x ``[B, H, N, D]`` torch tensor, cos/sin ``[B or 1, N, D]``; they are
+    unsqueezed at dim 1 like the reference's call (unsqueeze_dim=1).
+    """
+    import torch
+
+    x = x.cpu()
+    cos = cos.cpu().unsqueeze(1)
+    sin = sin.cpu().unsqueeze(1)
+    half = x.shape[-1] // 2
+    rot = torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+    return (x * cos) + (rot * sin)
+
+
+def rope_cos_sin(positions, head_dim: int, base: float = 10000.0, dtype=None):
+    """cos/sin tables ``[B, N, D]`` as LlamaRotaryEmbedding builds them (default rope type):
+    inv_freq = base^(-2i/D), freqs = pos * inv_freq in fp32, emb = cat(freqs, freqs), cast to dtype.
+    positions: integer tensor ``[B, N]``."""
+    import torch
+
+    inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
+    freqs = positions.cpu().float()[:, :, None] * inv_freq[None, None, :]
+    emb = torch.cat((freqs, freqs), dim=-1)
+    cos, sin = emb.cos(), emb.sin()
+    if dtype is not None:
+        cos, sin = cos.to(dtype), sin.to(dtype)
+    return cos, sin
+
