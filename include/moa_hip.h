@@ -89,7 +89,10 @@ size_t moa_decode_workspace_bytes(int B, int Hq, int Hkv, int D, int64_t sumC);
  * [B, sumC, D]; head_start, head_valid_len: int64 [B, Hkv].  The segments of
  * one batch row must not overlap (their lengths sum to at most sumC), as in
  * the packed cache; the workspace is sized for that.
- * This build covers Hq == Hkv, D in {64,128}, f16/bf16.
+ * Query head h reads ring h / (Hq/Hkv): grouped-query attention, which the
+ * reference does not have (its caller asserts one kv group,
+ * MoA/models/llama/modeling_llama.py:220-224), with Hq/Hkv in {1,2,4,8}.
+ * D in {64,128}, f16/bf16, at most 256 kv heads.
  */
 int moa_decode_fwd(const void* q, const void* kc, const void* vc, void* o,
                    void* workspace, size_t workspace_bytes,

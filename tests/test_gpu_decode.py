@@ -180,6 +180,49 @@ def test_decode_config_scale(dev):
     torch.testing.assert_close(out[:2].float(), dense.float(), rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("G", [2, 4, 8])
+@pytest.mark.parametrize("D", [128, 64])
+def test_grouped_query_decode(dev, dtype, G, D):
+    """G query heads per ring (not in the reference, whose caller asserts one kv group,
+    MoA/models/llama/modeling_llama.py:220-224): query head h reads ring h // G, like the prefill
+    kernel and the oracle's decode_segments(group=G)."""
+    from moa_amd import mixture_of_sparse_attention
+    rng = np.random.default_rng(100 * G + D)
+    sizes = [64, 576, 1344, 192, 2112, 35]
+    B, Hkv = 2, len(sizes)
+    _, kc, vc, hs, hv = _case(rng, B, sizes, D, dtype, dev, fill="partial")
+    hv[0, 1] = 0                                   # an empty ring: its G outputs are zero
+    q = torch.from_numpy(rng.standard_normal((B, Hkv * G, 1, D)).astype(np.float32)).to(dev, dtype)
+    out = mixture_of_sparse_attention(q, kc, vc, D ** -0.5, head_start_index=torch.from_numpy(hs).to(dev),
+                                      head_valid_length=torch.from_numpy(hv).to(dev))
+    assert out.shape == (B, 1, Hkv * G, D)
+    ref = decode_segments(q[:, :, 0].float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(),
+                          hs, hv, D ** -0.5, group=G)
+    _close(out[:, 0].float().cpu().numpy(), ref, ("gqa", G, D, dtype))
+    assert not out[0, 0, G:2 * G].any()
+    # the same rings read by one query head each (G = 1) give the same rows
+    for g in (0, G - 1):
+        q1 = q[:, g::G].contiguous()
+        out1 = mixture_of_sparse_attention(q1, kc, vc, D ** -0.5, head_start_index=torch.from_numpy(hs).to(dev),
+                                           head_valid_length=torch.from_numpy(hv).to(dev))
+        assert torch.equal(out1[:, 0], out[:, 0, g::G])
+
+
+def test_grouped_query_70b_shape(dev):
+    """The 70B shape of the largest config: 64 query heads on 8 rings, head_dim 128, B = 4."""
+    from moa_amd import mixture_of_sparse_attention
+    rng = np.random.default_rng(5)
+    sizes = [4096, 1024, 8192, 2048, 6144, 512, 3072, 7168]
+    q_, kc, vc, hs, hv = _case(rng, 4, sizes, 128, torch.bfloat16, dev)
+    q = torch.from_numpy(rng.standard_normal((4, 64, 1, 128)).astype(np.float32)).to(dev, torch.bfloat16)
+    out = mixture_of_sparse_attention(q, kc, vc, 128 ** -0.5, head_start_index=torch.from_numpy(hs).to(dev),
+                                      head_valid_length=torch.from_numpy(hv).to(dev))
+    ref = decode_segments(q[:, :, 0].float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(),
+                          hs, hv, 128 ** -0.5, group=8)
+    _close(out[:, 0].float().cpu().numpy(), ref, "70b")
+
+
 def test_errors(dev):
     from moa_amd import mixture_of_sparse_attention
     q = torch.zeros(1, 2, 1, 128, dtype=torch.float32, device=dev)
@@ -195,3 +238,9 @@ def test_errors(dev):
     k96 = torch.zeros(1, 256, 96, dtype=torch.float16, device=dev)
     with pytest.raises(NotImplementedError):  # head_dim 96 is not covered
         mixture_of_sparse_attention(q96, k96, k96, 1.0, head_start_index=hs, head_valid_length=hv)
+    q6 = torch.zeros(1, 6, 1, 128, dtype=torch.float16, device=dev)
+    with pytest.raises(NotImplementedError):  # 3 query heads per ring is not covered
+        mixture_of_sparse_attention(q6, k.half(), k.half(), 1.0, head_start_index=hs, head_valid_length=hv)
+    q3 = torch.zeros(1, 3, 1, 128, dtype=torch.float16, device=dev)
+    with pytest.raises(AssertionError):       # 3 query heads do not divide over 2 rings
+        mixture_of_sparse_attention(q3, k.half(), k.half(), 1.0, head_start_index=hs, head_valid_length=hv)
