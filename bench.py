@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--prefill-iters", type=int, default=10)
-    ap.add_argument("--only", choices=["decode", "prefill", "copy"], default=None,
+    ap.add_argument("--only", choices=["decode", "prefill", "copy", "e2e"], default=None,
                     help="profiling aid: run one part only and print its figures (not the contract line)")
     return ap.parse_args()
 
@@ -196,6 +196,49 @@ def bench_rope_append(torch, dev, args, cache, iters=50):
             "GB/s": nbytes / (fused_us * 1e-6) / 1e9}
 
 
+def bench_e2e(torch, dev, args, batch=8, n_ctx=16384, new_tokens=32):
+    """The attention path of a 7B-shaped decoder end to end (32 layers, hidden 4096, 32 heads of
+    128): q/k/v/o projections (library GEMMs), rotary embedding + cache update, sparse prefill of an
+    n_ctx-token prompt, then new_tokens decode steps.  Norms, MLPs and the LM head are not on the path
+    and are left out.  Random weights, synthetic plan (elastic spans)."""
+    from moa_amd.models.llama.modeling_llama import LlamaMixtureAttentionStack
+    from moa_amd.workloads import elastic_spans
+
+    L, hidden, H, D = args.layers, 4096, 32, 128
+    dtype = torch.float16
+    model = LlamaMixtureAttentionStack(L, hidden, H, head_dim=D, dtype=dtype, device=dev)
+    for p in model.parameters():
+        p.data.normal_(0.0, hidden ** -0.5)
+    # a plan whose cache sizes are sink (64) + the elastic window at n_ctx
+    plan = {"alphas": [[64 + s for s in elastic_spans(H, n_ctx, seed=l)] for l in range(L)],
+            "betas": [[0.0] * H for _ in range(L)]}
+    model.set_mixture_of_attention(plan, permute_head=True, moa_max_new_token=new_tokens)
+    gen = torch.Generator(device=dev).manual_seed(3)
+    x = torch.randn(batch, n_ctx, hidden, generator=gen, device=dev, dtype=dtype)
+    pos = torch.arange(n_ctx, device=dev)[None, :]
+    times = []
+    for _ in range(2):   # first pass warms up
+        cache = model.new_cache(batch, n_ctx, dev)
+        torch.cuda.synchronize(dev)
+        t0 = time.perf_counter()
+        h = model(x, pos, cache)
+        torch.cuda.synchronize(dev)
+        times.append(time.perf_counter() - t0)
+    prefill_s = times[-1]
+    x1 = h[:, -1:, :].contiguous()
+    for t in range(3):
+        model(x1, torch.full((1, 1), n_ctx + t, device=dev), cache)
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    for t in range(3, new_tokens):
+        model(x1, torch.full((1, 1), n_ctx + t, device=dev), cache)
+    torch.cuda.synchronize(dev)
+    dec_s = (time.perf_counter() - t0) / (new_tokens - 3)
+    return {"workload": f"attention path of a 7B-shaped decoder: L={L}, B={batch}, prompt {n_ctx}, fp16",
+            "prefill_s": prefill_s, "prefill_tokens_per_s": batch * n_ctx / prefill_s,
+            "decode_ms_per_step": dec_s * 1e3, "decode_tokens_per_s": batch / dec_s}
+
+
 def bench_prefill(torch, dev, args):
     from moa_amd import mixture_of_sparse_attention
     from moa_amd.workloads import elastic_spans, prefill_work
@@ -303,6 +346,9 @@ def main():
             y.copy_(x)
         torch.cuda.synchronize(dev)
         print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n, "launches": 5}))
+        return
+    if args.only == "e2e":
+        print(json.dumps({"e2e": bench_e2e(torch, dev, args)}))
         return
     if args.only == "prefill":
         print(json.dumps({"prefill": bench_prefill(torch, dev, args)}))

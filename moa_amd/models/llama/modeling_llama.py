@@ -1,0 +1,143 @@
+"""The caller of the attention path: a Llama-shaped attention layer that runs on moa_amd's kernels.
+
+Mirrors ``LlamaMixtureAttention.forward`` and ``LlamaModel.set_mixture_of_attention`` of the
+reference (MoA/models/llama/modeling_llama.py:206-332 and :334-406) without depending on a
+particular transformers version: the projections are ``torch.nn.Linear`` (rocBLAS/hipBLASLt GEMMs,
+outside the accelerated path), everything between them goes through libmoa_hip.so:
+
+    q, k, v projections -> rotary embedding + cache update (one launch in decode)
+                        -> mixture_of_sparse_attention (sparse prefill / ring decode) -> o_proj
+
+Unlike the reference (which asserts one key-value group, :220-224) grouped-query attention is
+accepted: the cache and the sparsity plan are per kv head.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+from torch import Tensor, nn
+
+from moa_amd.attention.cache_utils import StaticCircularCache, moa_config_to_cache_config
+from moa_amd.attention.permutation_utils import (moa_config_to_permutation, permute_attention_projection,
+                                                 permute_output_projection)
+from moa_amd.kernels.mixture_of_attention import mixture_of_sparse_attention
+
+
+def rotary_cos_sin(position_ids: Tensor, head_dim: int, dtype: torch.dtype, base: float = 10000.0
+                   ) -> Tuple[Tensor, Tensor]:
+    """cos/sin ``[batch, seq_len, head_dim]`` of the default Llama rotary embedding
+    (inv_freq = base^(-2i/d) in fp32, emb = cat(freqs, freqs), cast to ``dtype``)."""
+    dev = position_ids.device
+    inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.int64, device=dev).float() / head_dim))
+    freqs = position_ids.float()[:, :, None] * inv_freq[None, None, :]
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return emb.cos().to(dtype), emb.sin().to(dtype)
+
+
+class LlamaMixtureAttention(nn.Module):
+    """One attention layer.  ``forward`` follows the reference's (:232-326)."""
+
+    def __init__(self, hidden_size: int, num_heads: int, num_key_value_heads: Optional[int] = None,
+                 head_dim: Optional[int] = None, layer_idx: int = 0, bias: bool = False,
+                 dtype: torch.dtype = torch.float16, device=None):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.num_key_value_heads = num_key_value_heads or num_heads
+        assert num_heads % self.num_key_value_heads == 0
+        self.num_key_value_groups = num_heads // self.num_key_value_heads
+        self.head_dim = head_dim or hidden_size // num_heads
+        self.layer_idx = layer_idx
+        kw = dict(bias=bias, dtype=dtype, device=device)
+        self.q_proj = nn.Linear(hidden_size, num_heads * self.head_dim, **kw)
+        self.k_proj = nn.Linear(hidden_size, self.num_key_value_heads * self.head_dim, **kw)
+        self.v_proj = nn.Linear(hidden_size, self.num_key_value_heads * self.head_dim, **kw)
+        self.o_proj = nn.Linear(num_heads * self.head_dim, hidden_size, **kw)
+
+    def forward(self, hidden_states: Tensor, position_embeddings: Tuple[Tensor, Tensor],
+                past_key_value: StaticCircularCache, attention_mask: Optional[Tensor] = None) -> Tensor:
+        """hidden_states ``[batch, q_len, hidden]``; position_embeddings ``(cos, sin)`` each
+        ``[batch or 1, q_len, head_dim]``; attention_mask ``[batch, kv_len]`` of 0/1 marks left
+        padding of a prompt.  Returns ``[batch, q_len, hidden]``."""
+        assert not self.training, "only support inference now"
+        assert isinstance(past_key_value, StaticCircularCache)
+        bsz, q_len, _ = hidden_states.shape
+        # [B, q_len, H*D] viewed as [B, H, q_len, D]: no copy, the kernels take the strides
+        q = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
+        k = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+        v = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+        cos, sin = position_embeddings
+        q, keys, values = past_key_value.rope_update(q, k, v, cos, sin, self.layer_idx, attention_mask)
+        li = self.layer_idx
+        attn = mixture_of_sparse_attention(
+            q, keys, values, sm_scale=self.head_dim ** -0.5, attention_dropout=0.0,
+            sink_size=past_key_value.static_cache_size[li],
+            local_size=past_key_value.circular_cache_size[li],
+            head_start_index=past_key_value.cache_head_start_index[li],
+            head_valid_length=past_key_value.cache_valid_length[li],
+        )   # [batch, q_len, heads, head_dim]
+        return self.o_proj(attn.reshape(bsz, q_len, self.num_heads * self.head_dim))
+
+
+class LlamaMixtureAttentionStack(nn.Module):
+    """The attention path of a decoder: ``num_layers`` attention layers with residual
+    connections (norms and MLPs are not on the path and are left out).  Carries what
+    ``set_mixture_of_attention`` sets up in the reference: the plan, the optional head
+    permutation, and the cache built from the plan."""
+
+    def __init__(self, num_layers: int, hidden_size: int, num_heads: int,
+                 num_key_value_heads: Optional[int] = None, head_dim: Optional[int] = None,
+                 rope_base: float = 10000.0, dtype: torch.dtype = torch.float16, device=None):
+        super().__init__()
+        self.layers = nn.ModuleList(
+            LlamaMixtureAttention(hidden_size, num_heads, num_key_value_heads, head_dim, layer_idx=i, dtype=dtype,
+                                  device=device) for i in range(num_layers))
+        self.rope_base = rope_base
+        self.dtype = dtype
+        self.use_moa = False
+        self.moa_config: Optional[Dict] = None
+        self.moa_max_new_token = 1024
+        self.eval()
+
+    def set_mixture_of_attention(self, moa_config: Dict, permute_head: bool = False,
+                                 moa_max_new_token: int = 1024) -> None:
+        """Stores the plan (``alphas``/``betas`` per layer and kv head) and, with ``permute_head``,
+        clusters heads with equal (alpha, beta): the plan and the q/k/v/o projections of every
+        layer are re-ordered consistently (reference :373-398), which leaves the layer's function
+        unchanged."""
+        alphas = [list(a) for a in moa_config["alphas"]]
+        betas = [list(b) for b in moa_config["betas"]]
+        assert len(alphas) == len(self.layers) and len(betas) == len(self.layers)
+        if permute_head:
+            permutations, _ = moa_config_to_permutation({"alphas": alphas, "betas": betas})
+            for layer, perm in zip(self.layers, permutations):
+                i = layer.layer_idx
+                alphas[i] = [alphas[i][j] for j in perm.tolist()]
+                betas[i] = [betas[i][j] for j in perm.tolist()]
+                hk, g = layer.num_key_value_heads, layer.num_key_value_groups
+                permute_attention_projection(layer.q_proj, perm, hk, g)
+                permute_attention_projection(layer.k_proj, perm, hk)
+                permute_attention_projection(layer.v_proj, perm, hk)
+                permute_output_projection(layer.o_proj, perm, hk, g)
+        self.moa_config = {"alphas": alphas, "betas": betas}
+        self.moa_max_new_token = moa_max_new_token
+        self.use_moa = True
+
+    def new_cache(self, batch_size: int, seq_len: int, device) -> StaticCircularCache:
+        """The cache the reference's model forward builds at the start of a generation
+        (modeling_llama.py:93-112): sizes from the plan at this prompt length."""
+        assert self.use_moa, "call set_mixture_of_attention first"
+        cfg = moa_config_to_cache_config(self.moa_config, seq_len, max_new_token=self.moa_max_new_token,
+                                         sink_size=64, minimum_cache_size=128, split_size=64, verbose=False)
+        return StaticCircularCache(cache_size=cfg["cache_size"], static_size=cfg["static_size"],
+                                   batch_size=batch_size, head_dim=self.layers[0].head_dim, device=device,
+                                   dtype=self.dtype)
+
+    @torch.no_grad()
+    def forward(self, hidden_states: Tensor, position_ids: Tensor, past_key_value: StaticCircularCache,
+                attention_mask: Optional[Tensor] = None) -> Tensor:
+        cos, sin = rotary_cos_sin(position_ids, self.layers[0].head_dim, self.dtype, self.rope_base)
+        for layer in self.layers:
+            hidden_states = hidden_states + layer(hidden_states, (cos, sin), past_key_value, attention_mask)
+        return hidden_states
