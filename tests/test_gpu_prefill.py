@@ -125,6 +125,46 @@ def test_gqa(dev):
     _close(out, ref, "gqa")
 
 
+def test_many_heads_with_equal_and_extreme_spans(dev):
+    """The span-sorted work schedule: 40 heads (13B shape, not a multiple of the 8 XCDs) with tied
+    spans, heads that see nothing, heads wider than the prompt and block counts far out of range;
+    every head against the oracle, and the result must not depend on the order of the heads."""
+    B, H, N, D = 1, 40, 640, 64
+    nb = N // 64
+    rng = np.random.default_rng(11)
+    ns = [int(x) for x in rng.integers(0, 3, size=H)]
+    nl = [int(x) for x in rng.choice([0, 1, 2, 2, 2, 5, 5, nb, nb + 7], size=H)]
+    ns[3], nl[3] = 0, 0
+    q, k, v = _qkv(B, H, N, D, torch.float16, dev, seed=12)
+    out = _run(q, k, v, D ** -0.5, ns, nl, dev)
+    ref = prefill_masked_dense(q, k, v, D ** -0.5, ns, nl)
+    _close(out, ref, "many heads")
+    assert not out[:, 3].any()
+    perm = [int(x) for x in rng.permutation(H)]
+    outp = _run(q[:, perm], k[:, perm], v[:, perm], D ** -0.5, [ns[i] for i in perm], [nl[i] for i in perm], dev)
+    assert torch.equal(outp, out[:, perm])
+    # counts beyond the prompt (and negative ones) select the same tiles as their clamped values
+    from moa_amd.kernels.mixture_of_attention import moa_prefill
+    big = torch.tensor([10 ** 12 if n >= nb else n for n in nl], dtype=torch.int64, device=dev)
+    neg = torch.tensor([-5 if n == 0 else n for n in ns], dtype=torch.int64, device=dev)
+    out2 = moa_prefill(q.transpose(1, 2), k, v, num_global_blocks=neg, num_band_blocks=big, sm_scale=D ** -0.5)
+    assert torch.equal(out2.transpose(1, 2), out)
+
+
+def test_gqa_70b_shape(dev):
+    """The largest config's head layout: 64 query heads on 8 kv heads, head_dim 128, bf16 (its
+    32k-token prompt shortened to 4096 so that the CPU oracle finishes in seconds)."""
+    B, Hq, Hkv, N, D = 1, 64, 8, 4096, 128
+    q, k, v = _qkv(B, Hq, N, D, torch.bfloat16, dev, seed=13, hkv=Hkv)
+    ns, nl = [1] * Hkv, [4, 9, 17, 33, 2, 64, 12, 25]
+    out = _run(q, k, v, D ** -0.5, ns, nl, dev)
+    for hk in (0, 3, 5):
+        sl = slice(hk * 8, hk * 8 + 8)
+        ref = prefill_masked_dense(q[:, sl], k[:, hk:hk + 1].repeat_interleave(8, dim=1),
+                                   v[:, hk:hk + 1].repeat_interleave(8, dim=1), D ** -0.5, [ns[hk]] * 8, [nl[hk]] * 8)
+        _close(out[:, sl], ref, ("70b", hk))
+
+
 def test_short_prompt_falls_back_to_dense(dev):
     """N <= 64: dense causal with a warning (mixture_of_attention.py:412-415), whatever the spans."""
     from moa_amd import mixture_of_sparse_attention
