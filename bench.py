@@ -49,7 +49,7 @@ def parse_args():
     ap.add_argument("--ctx", type=int, default=16384)
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--prefill-iters", type=int, default=10)
+    ap.add_argument("--prefill-iters", type=int, default=20)
     ap.add_argument("--only", choices=["decode", "prefill", "copy", "e2e"], default=None,
                     help="profiling aid: run one part only and print its figures (not the contract line)")
     return ap.parse_args()
@@ -253,7 +253,7 @@ def bench_prefill(torch, dev, args):
     q, k, v = (torch.randn(B, N, H, D, generator=gen, device=dev, dtype=dtype).transpose(1, 2) for _ in range(3))
     sm = D ** -0.5
     flops, tile_flops, tiles = prefill_work(N, [1] * H, [s // 64 for s in spans], B, D)
-    for _ in range(2):
+    for _ in range(5):
         mixture_of_sparse_attention(q, k, v, sm, sink_size=sink, local_size=local)
     torch.cuda.synchronize(dev)
     evs = []

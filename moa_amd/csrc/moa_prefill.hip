@@ -97,15 +97,6 @@ struct PBF16 {
   }
 };
 
-// 4 consecutive rows of one 16-bit column out of a row-major LDS tile: within
-// each group of 16 lanes, lane i must point at (row0 + i/4, col0 + 4*(i%4));
-// it receives rows row0..row0+3 of column col0 + i.
-__device__ __forceinline__ u32x2 lds_read_tr16(const char* p) {
-  typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
-  s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
-  return __builtin_bit_cast(u32x2, r);
-}
-
 // Asynchronous 16-byte-per-lane copy global -> LDS (global_load_lds_dwordx4): lane i of the wave
 // reads base + byte_off(i) and lands at LDS byte address lds_addr + 16*i.  base and lds_addr are
 // wave-uniform.  Written as inline assembly on purpose: the compiler cannot prove that these LDS
@@ -151,8 +142,6 @@ __device__ __forceinline__ void phase_barrier() {
   asm volatile("" ::: "memory");
 }
 
-
-
 struct Strides4 {
   int64_t b, h, n;
 };
@@ -168,6 +157,9 @@ __device__ __forceinline__ u32x4 lds_load16(uint32_t addr, int imm) {
   typedef u32x4 __attribute__((address_space(3))) * lds_u32x4_ptr;
   return *(lds_u32x4_ptr)(uintptr_t)(addr + imm);
 }
+// The transposing read: 4 consecutive rows of one 16-bit column out of a row-major LDS tile.  Within
+// each group of 16 lanes, lane i must point at (row0 + i/4, col0 + 4*(i%4)); it receives rows
+// row0..row0+3 of column col0 + i.
 __device__ __forceinline__ u32x2 lds_load_tr16(uint32_t addr, int imm) {
   typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
   s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(uintptr_t)(addr + imm));
