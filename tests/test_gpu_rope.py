@@ -140,6 +140,40 @@ def test_fused_step_feeds_the_decode_kernel(dev):
         assert np.all(np.abs(got - ref) <= 2e-3 + 1e-2 * np.abs(ref)), t
 
 
+def test_fused_qkv_projection_buffer(dev):
+    """q, k and v as views of ONE fused projection output [B, q_len, (Hq + 2 Hkv) D] (the QKV split
+    costs no copy: the entry points take strides), prompt and decode step."""
+    from moa_amd import StaticCircularCache
+    dtype, B, Hq, Hkv, D, S = torch.bfloat16, 2, 8, 2, 64, 130
+    cache_size, static = [128, 192], [64, 64]
+    cache = StaticCircularCache([cache_size], static_size=[static], batch_size=B, head_dim=D, device=dev, dtype=dtype)
+    o = StaticCircularCacheOracle(cache_size, static, B, D)
+
+    def split(qkv):
+        n = qkv.shape[1]
+        q = qkv[..., : Hq * D].view(B, n, Hq, D).transpose(1, 2)
+        k = qkv[..., Hq * D: (Hq + Hkv) * D].view(B, n, Hkv, D).transpose(1, 2)
+        v = qkv[..., (Hq + Hkv) * D:].view(B, n, Hkv, D).transpose(1, 2)
+        return q, k, v
+
+    for step, n in enumerate([S, 1, 1]):
+        qkv = _rand((B, n, (Hq + 2 * Hkv) * D), dtype, 40 + step)
+        pos = torch.arange(n)[None, :] + (0 if step == 0 else S + step - 1)
+        cos, sin = rope_cos_sin(pos, D, dtype=dtype)
+        q, k, v = split(qkv)
+        qe, kk, vv = cache.rope_update(*split(qkv.to(dev)), cos.to(dev), sin.to(dev), 0)
+        assert _same_bits(qe, rope_reference(q, cos, sin)), step
+        k_ref = rope_reference(k, cos, sin).float().numpy()
+        if step == 0:
+            o.update_prefill(k_ref, v.float().numpy())
+        else:
+            o.update_decode(k_ref, v.float().numpy())
+        m = o.mask_cache == 1
+        assert np.array_equal(cache.key_cache[0].float().cpu().numpy()[m], o.key_cache[m]), step
+        assert np.array_equal(cache.value_cache[0].float().cpu().numpy()[m], o.value_cache[m]), step
+        assert cache.cache_update_index[0].cpu().numpy().tolist() == o.cache_update_index.tolist(), step
+
+
 def test_rope_errors(dev):
     from moa_amd import _lib
     from moa_amd.kernels.rotary import apply_rotary_pos_emb
