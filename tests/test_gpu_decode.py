@@ -223,6 +223,22 @@ def test_grouped_query_70b_shape(dev):
     _close(out[:, 0].float().cpu().numpy(), ref, "70b")
 
 
+def test_maximum_head_count(dev):
+    """256 rings per batch row is the limit of the chunk table; one more is refused."""
+    from moa_amd import mixture_of_sparse_attention
+    rng = np.random.default_rng(31)
+    sizes = [int(x) for x in rng.choice([64, 128, 576], size=256)]
+    q, kc, vc, hs, hv = _case(rng, 2, sizes, 64, torch.float16, dev, fill="partial")
+    out, ref = _run(q, kc, vc, hs, hv, 0.125, dev)
+    _close(out, ref, "256 heads")
+    q2 = torch.zeros(1, 257, 1, 64, dtype=torch.float16, device=dev)
+    k2 = torch.zeros(1, 257 * 64, 64, dtype=torch.float16, device=dev)
+    hs2 = (torch.arange(257, device=dev) * 64)[None, :]
+    hv2 = torch.full((1, 257), 64, device=dev)
+    with pytest.raises(NotImplementedError):
+        mixture_of_sparse_attention(q2, k2, k2, 0.125, head_start_index=hs2, head_valid_length=hv2)
+
+
 def test_errors(dev):
     from moa_amd import mixture_of_sparse_attention
     q = torch.zeros(1, 2, 1, 128, dtype=torch.float32, device=dev)

@@ -165,6 +165,18 @@ def test_gqa_70b_shape(dev):
         _close(out[:, sl], ref, ("70b", hk))
 
 
+def test_more_heads_than_the_sorted_schedule_covers(dev):
+    """Beyond 512 kv heads the span sort is skipped and heads are taken in the given order."""
+    B, H, N, D = 1, 520, 128, 64
+    rng = np.random.default_rng(21)
+    ns = [int(x) for x in rng.integers(0, 2, size=H)]
+    nl = [int(x) for x in rng.integers(0, 3, size=H)]
+    q, k, v = _qkv(B, H, N, D, torch.float16, dev, seed=22)
+    out = _run(q, k, v, D ** -0.5, ns, nl, dev)
+    ref = prefill_masked_dense(q, k, v, D ** -0.5, ns, nl)
+    _close(out, ref, "520 heads")
+
+
 def test_short_prompt_falls_back_to_dense(dev):
     """N <= 64: dense causal with a warning (mixture_of_attention.py:412-415), whatever the spans."""
     from moa_amd import mixture_of_sparse_attention
