@@ -177,6 +177,21 @@ def test_more_heads_than_the_sorted_schedule_covers(dev):
     _close(out, ref, "520 heads")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_peaked_and_drifting_scores(dev, dtype):
+    """Scores in the hundreds (one-hot-like softmax) and a row maximum that keeps growing along the
+    keys, so that the lazily updated softmax reference is rescaled many times."""
+    B, H, N, D = 1, 4, 768, 128
+    q, k, v = _qkv(B, H, N, D, dtype, dev, seed=31)
+    q = (q * 6).contiguous()
+    ramp = torch.linspace(0.2, 3.0, N, device=dev)[None, None, :, None]
+    k = (k * ramp.to(dtype)).contiguous()          # later keys are larger: the running max drifts upward
+    ns, nl = [1, 0, 2, 1], [12, 3, 5, 1]
+    out = _run(q, k, v, D ** -0.5, ns, nl, dev)
+    ref = prefill_masked_dense(q, k, v, D ** -0.5, ns, nl)
+    _close(out, ref, ("peaked", dtype))
+
+
 def test_short_prompt_falls_back_to_dense(dev):
     """N <= 64: dense causal with a warning (mixture_of_attention.py:412-415), whatever the spans."""
     from moa_amd import mixture_of_sparse_attention
