@@ -226,17 +226,38 @@ def bench_e2e(torch, dev, args, batch=8, n_ctx=16384, new_tokens=32):
         times.append(time.perf_counter() - t0)
     prefill_s = times[-1]
     x1 = h[:, -1:, :].contiguous()
-    for t in range(3):
-        model(x1, torch.full((1, 1), n_ctx + t, device=dev), cache)
+    pos1 = torch.full((1, 1), n_ctx, device=dev, dtype=torch.int64)
+
+    def step():
+        y = model(x1, pos1, cache)
+        pos1.add_(1)
+        return y
+
+    for _ in range(3):
+        step()
     torch.cuda.synchronize(dev)
     t0 = time.perf_counter()
-    for t in range(3, new_tokens):
-        model(x1, torch.full((1, 1), n_ctx + t, device=dev), cache)
+    for _ in range(3, new_tokens):
+        step()
     torch.cuda.synchronize(dev)
     dec_s = (time.perf_counter() - t0) / (new_tokens - 3)
+    # the same step captured once in a HIP graph and replayed (the library only enqueues kernels;
+    # the position advances on the device)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    for _ in range(new_tokens):
+        graph.replay()
+    torch.cuda.synchronize(dev)
+    graph_s = (time.perf_counter() - t0) / new_tokens
     return {"workload": f"attention path of a 7B-shaped decoder: L={L}, B={batch}, prompt {n_ctx}, fp16",
             "prefill_s": prefill_s, "prefill_tokens_per_s": batch * n_ctx / prefill_s,
-            "decode_ms_per_step": dec_s * 1e3, "decode_tokens_per_s": batch / dec_s}
+            "decode_ms_per_step": dec_s * 1e3, "decode_tokens_per_s": batch / dec_s,
+            "graph_decode_ms_per_step": graph_s * 1e3, "graph_decode_tokens_per_s": batch / graph_s}
 
 
 def bench_prefill(torch, dev, args):
