@@ -50,6 +50,9 @@ def parse_args():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--prefill-iters", type=int, default=20)
+    ap.add_argument("--plan", default=None,
+                    help='with --only e2e: a plan file in the reference\'s JSON format {"alphas": [L][H], "betas": [L][H]} '
+                         "(e.g. tests/golden/plan_vicuna-7b-v1.5-16k_moa_alpha_beta.json) instead of the synthetic plan")
     ap.add_argument("--only", choices=["decode", "prefill", "copy", "e2e"], default=None,
                     help="profiling aid: run one part only and print its figures (not the contract line)")
     return ap.parse_args()
@@ -200,18 +203,26 @@ def bench_e2e(torch, dev, args, batch=8, n_ctx=16384, new_tokens=32):
     """The attention path of a 7B-shaped decoder end to end (32 layers, hidden 4096, 32 heads of
     128): q/k/v/o projections (library GEMMs), rotary embedding + cache update, sparse prefill of an
     n_ctx-token prompt, then new_tokens decode steps.  Norms, MLPs and the LM head are not on the path
-    and are left out.  Random weights, synthetic plan (elastic spans)."""
+    and are left out.  Random weights; the plan is synthetic (elastic spans) unless --plan names a
+    plan file, whose layer and head counts then set the shape (head dim stays 128)."""
     from moa_amd.models.llama.modeling_llama import LlamaMixtureAttentionStack
     from moa_amd.workloads import elastic_spans
 
-    L, hidden, H, D = args.layers, 4096, 32, 128
+    L, H, D = args.layers, 32, 128
+    plan = None
+    if args.plan:
+        with open(args.plan) as f:
+            plan = json.load(f)
+        L, H = len(plan["alphas"]), len(plan["alphas"][0])
+    hidden = H * D
     dtype = torch.float16
     model = LlamaMixtureAttentionStack(L, hidden, H, head_dim=D, dtype=dtype, device=dev)
     for p in model.parameters():
         p.data.normal_(0.0, hidden ** -0.5)
     # a plan whose cache sizes are sink (64) + the elastic window at n_ctx
-    plan = {"alphas": [[64 + s for s in elastic_spans(H, n_ctx, seed=l)] for l in range(L)],
-            "betas": [[0.0] * H for _ in range(L)]}
+    if plan is None:
+        plan = {"alphas": [[64 + s for s in elastic_spans(H, n_ctx, seed=l)] for l in range(L)],
+                "betas": [[0.0] * H for _ in range(L)]}
     model.set_mixture_of_attention(plan, permute_head=True, moa_max_new_token=new_tokens)
     gen = torch.Generator(device=dev).manual_seed(3)
     x = torch.randn(batch, n_ctx, hidden, generator=gen, device=dev, dtype=dtype)
@@ -254,7 +265,10 @@ def bench_e2e(torch, dev, args, batch=8, n_ctx=16384, new_tokens=32):
         graph.replay()
     torch.cuda.synchronize(dev)
     graph_s = (time.perf_counter() - t0) / new_tokens
-    return {"workload": f"attention path of a 7B-shaped decoder: L={L}, B={batch}, prompt {n_ctx}, fp16",
+    kept = sum(cache.layer_cache_size) / (L * H * (n_ctx + new_tokens))
+    return {"workload": f"attention path of a decoder: L={L}, H={H}, D={D}, B={batch}, prompt {n_ctx}, fp16",
+            "plan": os.path.basename(args.plan) if args.plan else "synthetic elastic spans",
+            "kv_kept_fraction": kept,
             "prefill_s": prefill_s, "prefill_tokens_per_s": batch * n_ctx / prefill_s,
             "decode_ms_per_step": dec_s * 1e3, "decode_tokens_per_s": batch / dec_s,
             "graph_decode_ms_per_step": graph_s * 1e3, "graph_decode_tokens_per_s": batch / graph_s}
