@@ -67,18 +67,10 @@ struct PF16 {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
-  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
-  }
-  static __device__ __forceinline__ uint32_t pack_rne(float lo, float hi) {
+  static __device__ __forceinline__ uint32_t pack_rne(float lo, float hi) {   // one v_cvt_pk_f16_f32
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
     h2 r = {(_Float16)lo, (_Float16)hi};
     return __builtin_bit_cast(uint32_t, r);
-  }
-  // acc + lo + hi of a packed pair (v_dot2_f32_f16 with a pair of ones)
-  static __device__ __forceinline__ float add_pair(uint32_t pk, float acc) {
-    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, pk), h2{(_Float16)1.f, (_Float16)1.f}, acc, false);
   }
 };
 struct PBF16 {
@@ -86,14 +78,9 @@ struct PBF16 {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
-  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+  static __device__ __forceinline__ uint32_t pack_rne(float lo, float hi) {   // one v_cvt_pk_bf16_f32
     f32x2 x = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2v));
-  }
-  static __device__ __forceinline__ uint32_t pack_rne(float lo, float hi) { return pack(lo, hi); }
-  // acc + lo + hi of a packed pair (v_dot2_f32_bf16 with a pair of ones)
-  static __device__ __forceinline__ float add_pair(uint32_t pk, float acc) {
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2v, pk), __builtin_bit_cast(bf16x2v, 0x3f803f80u), acc, false);
   }
 };
 
@@ -269,7 +256,6 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
   const int w_hi1 = min(ns - 1, mbw);
   const int w_lo2 = max(0, mbw + 1 - nl);
   auto live_tile = [&](int j) __attribute__((always_inline)) { return wave_has_rows && (j <= w_hi1 || (j >= w_lo2 && j <= mbw)); };
-  auto live = [&](int t) __attribute__((always_inline)) { return t >= 0 && t < n_tiles && live_tile(tile_at(t)); };
 
   const int64_t m_glob = (int64_t)qt * kQRows + wave * kWRows + mcol;   // this lane's query row
 
@@ -296,11 +282,13 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
   }
   // rows >= N of the ragged last tile repeat row N-1: their scores are masked, their softmax
   // weight is exactly 0, and a repeated real row is finite
-  auto issue_tile = [&](const uint16_t* base, int64_t stride_n, const uint32_t (&off)[LPW], bool is_k,
-                        int j, char* stage) {
-    const uint16_t* src = base + (int64_t)j * kKV * stride_n;
-    const uint32_t dst = lds_address(stage) + wave * LPW * 1024;
-    if ((j + 1) * kKV <= N) {
+  // a tile is 64 rows: its byte offset inside the head fits 32 bits (checked on the host)
+  const uint32_t k_tile_bytes = (uint32_t)(2 * kKV * ks.n), v_tile_bytes = (uint32_t)(2 * kKV * vs.n);
+  const int j_ragged = (N % kKV) ? nb - 1 : -1;    // the only tile with rows past N, if any
+  auto issue_tile = [&](const uint16_t* base, uint32_t tile_bytes, int64_t stride_n, const uint32_t (&off)[LPW],
+                        bool is_k, int j, uint32_t dst) __attribute__((always_inline)) {
+    const char* src = reinterpret_cast<const char*>(base) + (uint64_t)(uint32_t)j * tile_bytes;
+    if (j != j_ragged) {
 #pragma unroll
       for (int i = 0; i < LPW; ++i) async_copy16(src, off[i], dst + i * 1024);
     } else {
@@ -314,17 +302,32 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
       }
     }
   };
-  auto issue_k = [&](int t) __attribute__((always_inline)) { issue_tile(kbase, ks.n, koff, true, tile_at(t), s_k + (t % kStages) * TILE_B); };
-  auto issue_v = [&](int t) __attribute__((always_inline)) { issue_tile(vbase, vs.n, voff, false, tile_at(t), s_v + (t % kStages) * TILE_B); };
-  auto batch_size = [&](int s) __attribute__((always_inline)) { return (s < 0) ? 0 : ((s + 3 < n_tiles) ? LPW : 0) + ((s + 2 < n_tiles) ? LPW : 0); };
+  // Scalar schedule state.  The tile order is piecewise consecutive (sinks, then the band from its
+  // rotated start, wrapping once), so the tile of the next step follows from the current one with a
+  // few scalar instructions; a step past the last tile repeats the last tile: its copy goes into a
+  // stage that nobody reads any more, every iteration starts the same number of copies and the
+  // wait before a barrier is a constant.
+  const int band_last = lo2 + n_band - 1;
+  const int band_first = lo2 + band_rot;
+  auto next_tile = [&](int j, int t_next) __attribute__((always_inline)) {
+    int jn = j + 1;
+    jn = (jn > band_last) ? lo2 : jn;
+    jn = (t_next == n_sink) ? band_first : jn;
+    return (t_next >= n_tiles) ? j : jn;
+  };
+  constexpr uint32_t kRing = kStages * TILE_B;                       // bytes of one tensor's ring (a power of two)
+  const uint32_t k_dst0 = lds_address(s_k) + wave * LPW * 1024;      // this wave's share of stage 0
+  const uint32_t v_dst0 = lds_address(s_v) + wave * LPW * 1024;
+  int j_0 = tile_at(0), j_1 = next_tile(j_0, 1), j_2 = next_tile(j_1, 2), j_3 = next_tile(j_2, 3);   // tiles of steps t .. t+3
 
   // The matrix phase of iteration t reads K(t) and V(t-1) and starts the copies of K(t+3) and
   // V(t+2), whose stages were last read in iteration t-1 by both groups.  Before the loop:
   // K(0..2), V(0..1).
-  issue_k(0);
-  issue_v(0);
-  if (n_tiles > 1) { issue_k(1); issue_v(1); }
-  if (n_tiles > 2) issue_k(2);
+  issue_tile(kbase, k_tile_bytes, ks.n, koff, true, j_0, k_dst0);
+  issue_tile(vbase, v_tile_bytes, vs.n, voff, false, j_0, v_dst0);
+  issue_tile(kbase, k_tile_bytes, ks.n, koff, true, j_1, k_dst0 + TILE_B);
+  issue_tile(vbase, v_tile_bytes, vs.n, voff, false, j_1, v_dst0 + TILE_B);
+  issue_tile(kbase, k_tile_bytes, ks.n, koff, true, j_2, k_dst0 + 2 * TILE_B);
 
   // ---- Q fragment (B operand): Q[m][16*ks + 8*g .. +7] ---------------------
   u32x4 qf[KS];
@@ -433,14 +436,13 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
   // every P.V issued so far belongs to earlier tiles and has completed in this wave's matrix phase)
   auto softmax = [&](int j) __attribute__((always_inline)) {
     if (j == mbw) {   // causal mask on the diagonal tile
-      const int m_in = (wave & 1) * kWRows + mcol;   // row inside the 64-row block
+      int thr = (wave & 1) * kWRows + mcol - 4 * g;   // row inside the 64-row block, minus the lane's column base
+      asm volatile("" : "+v"(thr));                  // keeps the 32 compares in this branch instead of 32 hoisted lane masks
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int n_in = nt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-          if (n_in > m_in) st[nt][i] = -INFINITY;
-        }
+        for (int i = 0; i < 16; ++i)
+          if (nt * 32 + 8 * (i >> 2) + (i & 3) > thr) st[nt][i] = -INFINITY;
     }
     float mx = st[0][0];
 #pragma unroll
@@ -459,16 +461,19 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
         for (int i = 0; i < 16; ++i) oacc[t][i] *= alpha;
       m_run = m_new;
     }
-    float psum[2] = {0.f, 0.f};   // two chains: a dot2 result is not ready for the very next instruction
+    // Row sums are plain fp32 adds of the unrounded weights.  (v_dot2_f32_{f16,bf16} of the packed
+    // pair with a pair of ones would halve the instruction count, but those instructions stall the
+    // MFMA stream of the wave that shares the SIMD: measured 20 % slower per iteration.)
+    float psum[2] = {0.f, 0.f};
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int i = 0; i < 16; i += 2) {
         const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i], scale_log2, -m_run));
         const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i + 1], scale_log2, -m_run));
-        const uint32_t pk = T::pack(p0, p1);
-        pf[nt * 8 + (i >> 1)] = pk;
-        psum[(i >> 1) & 1] = T::add_pair(pk, psum[(i >> 1) & 1]);   // the sum of what P.V multiplies with: the rounded weights
+        pf[nt * 8 + (i >> 1)] = T::pack_rne(p0, p1);
+        psum[0] += p0;
+        psum[1] += p1;
       }
     l_run += psum[0] + psum[1];
   };
@@ -490,13 +495,17 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
   // barrier t-1; the copies started two iterations ago (K(t+1), V(t)) are first read after barrier
   // t, and every wave waits for its own before it.  Iteration n_tiles only finishes P.V of the
   // last tile.
+  uint32_t cst = 3 * TILE_B;   // ring offset of the stage K(t+3) is copied into; V(t+2) goes one stage below
+  uint32_t rst = 0;            // ring offset of the stage K(t) is read from
+  int kd_prev = 0;             // how far the K read addresses moved in the previous iteration
+  bool lc_prev = false;        // was tile t-1 live for this wave
   auto iteration = [&](int t, auto FIRST) __attribute__((always_inline)) {
     constexpr bool kFirst = decltype(FIRST)::value != 0;
-    const int n_wait = batch_size(t - 1) + batch_size(t);
+    constexpr int n_wait = 4 * LPW;   // the copies of this iteration and the one before may still be in flight
     // ---------------- matrix phase ----------------
-    if (t + 3 < n_tiles) issue_k(t + 3);
-    if (t + 2 < n_tiles) issue_v(t + 2);
-    const bool lp = live(t - 1), lc = live(t);
+    issue_tile(kbase, k_tile_bytes, ks.n, koff, true, j_3, k_dst0 + cst);
+    issue_tile(vbase, v_tile_bytes, vs.n, voff, false, j_2, v_dst0 + ((cst - TILE_B) & (kRing - 1)));
+    const bool lp = lc_prev, lc = (t < n_tiles) && live_tile(j_0);
     if (kFirst) {
       if (lc) qk_phase();
     } else {
@@ -505,27 +514,35 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
     if (grp == 1) { wait_vm(n_wait); phase_barrier(); }
     // ---------------- softmax phase ----------------
     if (lc) {
-      softmax(tile_at(t));
+      softmax(j_0);
     } else if (lp) {   // the next matrix phase this wave runs must add nothing for a dead tile
 #pragma unroll
       for (int i = 0; i < 16; ++i) pf[i] = 0;
     }
-    // advance the operand addresses to the next stages (K: t+1, V: t)
+    // advance the operand addresses to the next stages (K: t+1, V: t) and the schedule by one step
     {
-      const int kd = ((t + 1) % kStages == 0) ? -(kStages - 1) * TILE_B : TILE_B;
+      const int kd = (rst == (kStages - 1) * TILE_B) ? -(kStages - 1) * TILE_B : TILE_B;
 #pragma unroll
       for (int s = 0; s < KS; ++s) k_ad[s] += kd;
       if (!kFirst) {
-        const int vd = (t % kStages == 0) ? -(kStages - 1) * TILE_B : TILE_B;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) v_ad[dt] += vd;
+        for (int dt = 0; dt < DT; ++dt) v_ad[dt] += kd_prev;   // V trails K by one step
       }
+      kd_prev = kd;
+      rst = (rst + TILE_B) & (kRing - 1);
+      cst = (cst + TILE_B) & (kRing - 1);
+      lc_prev = lc;
+      j_0 = j_1;
+      j_1 = j_2;
+      j_2 = j_3;
+      j_3 = next_tile(j_3, t + 4);
     }
     if (grp == 0) { wait_vm(n_wait); phase_barrier(); }
   };
   iteration(0, IC<1>{});   // no P.V yet (and no V stage to read)
   for (int t = 1; t <= n_tiles; ++t) iteration(t, IC<0>{});
 
+  wait_vm(0);   // the repeated copies of the last steps
   // ---- epilogue: O[m][d] = O^T[d][m] / l ---------------------------------
   if (!wave_has_rows || m_glob >= N) return;
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
