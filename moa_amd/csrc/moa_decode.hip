@@ -25,7 +25,7 @@
 //   * grouped-query attention (G = Hq / Hkv query heads per ring, which the
 //     reference does not have): the G query rows of a ring share every K/V
 //     row that a wave loads, so the cache is still read once.
-#include "moa_common.h"
+#include "moa_mfma.h"
 
 #include <hip/hip_fp16.h>
 
@@ -333,6 +333,246 @@ __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
   }
 }
 
+
+// ---- grouped-query decode on the matrix cores (G >= 4) ---------------------------------------
+// With G query heads per ring the vector ALU version above does G times the arithmetic per cache
+// byte and stops being HBM bound (46 % of peak at G = 8).  Here the G query rows of a ring are the
+// columns of a 32-wide MFMA tile (columns >= G are zero padding; the matrix pipe has the room):
+//   S^T[key][q] = sum_d K[key][d] Q[q][d]      A = K (LDS), B = Q^T (registers)
+//   O^T[d][q]   = sum_key V[key][d] P[q][key]   A = V^T (LDS, transposing read), B = P^T
+// the same transposed pair of products as the prefill kernel, 32 keys at a time, so the softmax
+// state of a query head is lane-local.  Each wave streams its own share of the chunk through a
+// private two-stage LDS ring with asynchronous copies (16-byte chunks XOR-permuted as in the
+// prefill kernel), so no work-group barrier is needed inside the loop.  Chunks, partials and the
+// merge kernel are those of the vector version, with a longer chunk.
+constexpr int kGqaChunk = 1024;   // cache rows per work-group step (256 per wave)
+constexpr int kGqaTile = 32;      // keys per MFMA tile
+constexpr int kGqaStages = 2;     // LDS stages per wave
+
+template <typename T> struct MfmaElem;
+template <> struct MfmaElem<F16> { typedef PF16 type; };
+template <> struct MfmaElem<BF16> { typedef PBF16 type; };
+
+template <int D>
+constexpr size_t gqa_lds_bytes() { return (size_t)kDecWaves * kGqaStages * 2 * kGqaTile * D * 2; }
+
+template <typename T, int D, int G>
+__global__ __launch_bounds__(kDecThreads) void decode_gqa_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
+    uint16_t* __restrict__ o, float* __restrict__ part_acc, float* __restrict__ part_ml,
+    const int64_t* __restrict__ head_start, const int64_t* __restrict__ head_valid, int H,
+    int64_t sumC, float scale_log2, int cap) {
+  typedef typename MfmaElem<T>::type M;
+  constexpr int KS = D / 16;                    // MFMA k-steps of Q.K^T
+  constexpr int DT = D / 32;                    // 32-wide d tiles of the output
+  constexpr int CPR = D / 8;                    // 16-byte chunks per cache row
+  constexpr int ROW_B = D * 2;
+  constexpr int RSH = 16 / CPR;                 // rows per 256 bytes of LDS
+  constexpr int TILE_B = kGqaTile * ROW_B;      // bytes of one K or V tile
+  constexpr int NCP = TILE_B / 1024;            // async copies per tile and tensor
+  constexpr int STAGE_B = 2 * TILE_B;           // K tile, then V tile
+  constexpr int WCHUNK = kGqaChunk / kDecWaves;
+  constexpr float kRescaleStep = 8.f;
+
+  extern __shared__ __attribute__((aligned(1024))) char s_mem[];
+  __shared__ int s_prefix[kMaxHeads + 1];
+  __shared__ float s_acc[kDecWaves][G][D];
+  __shared__ float s_m[kDecWaves][G];
+  __shared__ float s_l[kDecWaves][G];
+
+  const int b = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int mcol = lane & 31;   // query head inside the ring (the MFMA column); >= G: padding
+  const int g = lane >> 5;      // half-wave
+  const uint32_t ring0 = lds_address(s_mem) + wave * (kGqaStages * STAGE_B);   // this wave's stages
+
+  // copy i of a tile moves chunks [64 i, 64 i + 64): chunk c = row * CPR + position
+  uint32_t koff[NCP], voff[NCP];
+  int crow[NCP];
+#pragma unroll
+  for (int i = 0; i < NCP; ++i) {
+    const int L = i * 64 + lane;
+    const int row = L / CPR, pos = L % CPR;
+    crow[i] = row;
+    koff[i] = (uint32_t)((pos ^ ((row / RSH) % CPR)) * 16);
+    voff[i] = (uint32_t)((pos ^ (4 * ((row / RSH) % (CPR / 4)))) * 16);
+  }
+  // operand read addresses inside stage 0 (see the prefill kernel for the layout)
+  uint32_t k_ad[KS], v_ad[DT];
+  {
+    const uint32_t k_rd = (uint32_t)(mcol * ROW_B) | (uint32_t)(((g ^ ((mcol / RSH) % CPR)) & (CPR - 1)) * 16);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) k_ad[s] = ring0 + (k_rd ^ (uint32_t)(32 * s));
+    const int grp16 = lane & 15, dhalf = (lane >> 4) & 1, v_row = 4 * g + (grp16 >> 2);
+    const uint32_t v_rd = (uint32_t)(v_row * ROW_B) +
+                          (uint32_t)(((2 * dhalf + ((grp16 & 3) >> 1)) ^ (4 * ((v_row / RSH) % (CPR / 4)))) * 16 +
+                                     8 * (grp16 & 1));
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) v_ad[dt] = ring0 + TILE_B + (v_rd ^ (uint32_t)(64 * dt));
+  }
+
+  const int total = min(build_prefix<kGqaChunk>(head_valid + (int64_t)b * H, H, s_prefix), cap);
+
+  for (int w = blockIdx.x; w < total; w += gridDim.x) {
+    const int h = find_head(s_prefix, H, w);
+    const int c = w - s_prefix[h];
+    const int n_chunks = s_prefix[h + 1] - s_prefix[h];
+    const int64_t bh = (int64_t)b * H + h;
+    const int64_t seg0 = head_start[bh];
+    int64_t len = head_valid[bh];
+    if (seg0 < 0 || seg0 >= sumC) len = 0;   // clamp the segment into the row so that a bad index cannot fault
+    if (len > sumC - seg0) len = sumC - seg0;
+    const int64_t r_begin = (int64_t)c * kGqaChunk + (int64_t)wave * WCHUNK;
+    int64_t r_end = r_begin + WCHUNK;
+    if (r_end > len) r_end = len;
+    const int n_rows = __builtin_amdgcn_readfirstlane(r_end > r_begin ? (int)(r_end - r_begin) : 0);
+    const int n_t = (n_rows + kGqaTile - 1) / kGqaTile;
+    const char* kbase = reinterpret_cast<const char*>(kc + ((int64_t)b * sumC + seg0 + r_begin) * D);
+    const char* vbase = reinterpret_cast<const char*>(vc + ((int64_t)b * sumC + seg0 + r_begin) * D);
+
+    // Q^T fragments: column mcol = query head, k-step s holds Q[mcol][16 s + 8 g .. +7]
+    u32x4 qf[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      u32x4 z = {0, 0, 0, 0};
+      qf[s] = (mcol < G) ? *reinterpret_cast<const u32x4*>(q + (bh * G + mcol) * D + 16 * s + 8 * g) : z;
+    }
+    f32x16 oacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+
+    // tile t: rows [32 t, 32 t + 32) of the wave's share, into stage t % kGqaStages; rows past the
+    // end repeat the last row (their scores are masked)
+    auto issue = [&](int t) __attribute__((always_inline)) {
+      const char* ksrc = kbase + (int64_t)t * TILE_B;
+      const char* vsrc = vbase + (int64_t)t * TILE_B;
+      const uint32_t dst = ring0 + (t % kGqaStages) * STAGE_B;
+      const int last = n_rows - 1 - t * kGqaTile;   // >= 0
+#pragma unroll
+      for (int i = 0; i < NCP; ++i) async_copy16(ksrc, (uint32_t)(min(crow[i], last) * ROW_B) + koff[i], dst + i * 1024);
+#pragma unroll
+      for (int i = 0; i < NCP; ++i) async_copy16(vsrc, (uint32_t)(min(crow[i], last) * ROW_B) + voff[i], dst + TILE_B + i * 1024);
+    };
+    if (n_t > 0) issue(0);
+    if (n_t > 1) issue(1);
+    // the Q loads are older than every copy: pin their arrival here
+    if (n_t > 1) wait_vm(4 * NCP); else if (n_t > 0) wait_vm(2 * NCP);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[s]));
+
+    for (int t = 0; t < n_t; ++t) {
+      if (t + 1 < n_t) wait_vm(2 * NCP); else wait_vm(0);     // tile t has landed; tile t+1 may be in flight
+      const uint32_t so = (uint32_t)((t % kGqaStages) * STAGE_B);
+      // ---- S^T = K . Q^T ----
+      f32x16 st;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) st[i] = 0.f;
+      {
+        u32x4 kf[KS];
+#pragma unroll
+        for (int s = 0; s < KS; ++s) kf[s] = lds_load16(k_ad[s] + so, 0);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) st = M::mfma(kf[s], qf[s], st);
+      }
+      // ---- softmax over the 32 keys (element i of a lane: key 8 (i / 4) + 4 g + i % 4) ----
+      const int n_valid = n_rows - t * kGqaTile;
+      if (n_valid < kGqaTile) {
+        int thr = n_valid - 4 * g;
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (8 * (i >> 2) + (i & 3) >= thr) st[i] = -INFINITY;
+      }
+      float mx = st[0];
+#pragma unroll
+      for (int i = 1; i < 16; ++i) mx = fmaxf(mx, st[i]);
+      mx = max_with_other_half(mx);
+      const float m_cand = mx * scale_log2;   // finite: key 0 of the tile is valid
+      if (__any(m_cand > m_run + kRescaleStep)) {
+        const float m_new = fmaxf(m_run, m_cand);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        l_run *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+        m_run = m_new;
+      }
+      uint32_t pf[8];
+      float psum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[i], scale_log2, -m_run));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[i + 1], scale_log2, -m_run));
+        pf[i >> 1] = M::pack_rne(p0, p1);
+        psum += p0 + p1;
+      }
+      l_run += psum;
+      // ---- O^T += V^T . P^T ----
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk) {
+        const u32x4 bfrag = {pf[4 * tk], pf[4 * tk + 1], pf[4 * tk + 2], pf[4 * tk + 3]};
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const u32x2 lo = lds_load_tr16(v_ad[dt] + so, (16 * tk) * ROW_B);
+          const u32x2 hi = lds_load_tr16(v_ad[dt] + so, (16 * tk + 8) * ROW_B);
+          oacc[dt] = M::mfma(u32x4{lo.x, lo.y, hi.x, hi.y}, bfrag, oacc[dt]);
+        }
+      }
+      if (t + kGqaStages < n_t) issue(t + kGqaStages);   // every read of this stage has returned
+    }
+
+    // ---- the wave's result per query head: (m, l, O[d]) ----
+    {
+      const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+      if (mcol < G) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s_acc[wave][mcol][32 * dt + 8 * (i >> 2) + 4 * g + (i & 3)] = oacc[dt][i];
+        if (g == 0) {
+          s_m[wave][mcol] = m_run;
+          s_l[wave][mcol] = l_tot;
+        }
+      }
+    }
+    __syncthreads();
+
+    // ---- combine the waves; thread d owns output column d of every query head of the ring ----
+    if (tid < D) {
+#pragma unroll
+      for (int gq = 0; gq < G; ++gq) {
+        float Mx = s_m[0][gq];
+#pragma unroll
+        for (int i = 1; i < kDecWaves; ++i) Mx = fmaxf(Mx, s_m[i][gq]);
+        const float m_use = (Mx == -INFINITY) ? 0.f : Mx;
+        float L = 0.f, a = 0.f;
+#pragma unroll
+        for (int i = 0; i < kDecWaves; ++i) {
+          const float f = fast_exp2(s_m[i][gq] - m_use);
+          L += s_l[i][gq] * f;
+          a += s_acc[i][gq][tid] * f;
+        }
+        if (n_chunks == 1) {
+          o[(bh * G + gq) * D + tid] = pack1<T>((L > 0.f) ? a / L : 0.f);
+        } else {
+          const int64_t slot = ((int64_t)b * cap + w) * G + gq;
+          part_acc[slot * D + tid] = a;
+          if (tid == 0) {
+            part_ml[slot * 2 + 0] = Mx;
+            part_ml[slot * 2 + 1] = L;
+          }
+        }
+      }
+    }
+    __syncthreads();  // s_acc / s_m / s_l are reused by the next chunk
+  }
+}
+
 #ifndef MOA_DEC_CHUNK
 #define MOA_DEC_CHUNK 512
 #endif
@@ -366,6 +606,37 @@ static int launch_decode(const void* q, const void* kc, const void* vc, void* o,
   constexpr int GROUPS = kDecThreads / D;
   int mx = (H * G + GROUPS - 1) / GROUPS;
   hipLaunchKernelGGL((decode_merge_kernel<T, D, kChunk, G>), dim3(mx, B), dim3(kDecThreads), 0, st,
+                     (uint16_t*)o, part_acc, part_ml, head_valid, H, cap);
+  return check_launch("moa_decode_fwd(merge)");
+}
+
+
+template <typename T, int D, int G>
+static int launch_decode_gqa(const void* q, const void* kc, const void* vc, void* o, float* part_acc,
+                             float* part_ml, const int64_t* head_start, const int64_t* head_valid, int B,
+                             int H, int64_t sumC, float sm_scale, hipStream_t st) {
+  const int cap = (int)decode_cap(sumC, H);   // partial slots per batch row the workspace was sized for
+  const int64_t chunks = (sumC + kGqaChunk - 1) / kGqaChunk + H;   // at most this many steps per batch row
+  int bx = (int)((256 * 4 + B - 1) / B);   // one work-group per CU at a time (its LDS ring fills the CU)
+  if (bx > chunks) bx = (int)chunks;
+  if (bx < 1) bx = 1;
+  constexpr size_t lds = gqa_lds_bytes<D>();
+  static bool attr_set = false;   // per template instance
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_gqa_kernel<T, D, G>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess)
+      return fail(MOA_ERR_LAUNCH, "moa_decode_fwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((decode_gqa_kernel<T, D, G>), dim3(bx, B), dim3(kDecThreads), lds, st,
+                     (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, (uint16_t*)o,
+                     part_acc, part_ml, head_start, head_valid, H, sumC, sm_scale * kLog2e, cap);
+  int rc = check_launch("moa_decode_fwd(grouped split)");
+  if (rc) return rc;
+  constexpr int GROUPS = kDecThreads / D;
+  int mx = (H * G + GROUPS - 1) / GROUPS;
+  hipLaunchKernelGGL((decode_merge_kernel<T, D, kGqaChunk, G>), dim3(mx, B), dim3(kDecThreads), 0, st,
                      (uint16_t*)o, part_acc, part_ml, head_valid, H, cap);
   return check_launch("moa_decode_fwd(merge)");
 }
@@ -410,8 +681,8 @@ extern "C" int moa_decode_fwd(const void* q, const void* kc, const void* vc, voi
   switch (G) {                                                  \
     case 1: return launch_decode<T, DD, 1>(MOA_DEC_ARGS);       \
     case 2: return launch_decode<T, DD, 2>(MOA_DEC_ARGS);       \
-    case 4: return launch_decode<T, DD, 4>(MOA_DEC_ARGS);       \
-    default: return launch_decode<T, DD, 8>(MOA_DEC_ARGS);      \
+    case 4: return launch_decode_gqa<T, DD, 4>(MOA_DEC_ARGS);   \
+    default: return launch_decode_gqa<T, DD, 8>(MOA_DEC_ARGS);  \
   }
   if (dtype == MOA_DTYPE_F16) {
     if (D == 128) { MOA_DEC_G(F16, 128) }

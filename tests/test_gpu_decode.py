@@ -201,12 +201,13 @@ def test_grouped_query_decode(dev, dtype, G, D):
                           hs, hv, D ** -0.5, group=G)
     _close(out[:, 0].float().cpu().numpy(), ref, ("gqa", G, D, dtype))
     assert not out[0, 0, G:2 * G].any()
-    # the same rings read by one query head each (G = 1) give the same rows
+    # the same rings read by one query head each (G = 1, the vector-ALU kernel; G >= 4 runs on the
+    # matrix cores with P rounded to the input type) give the same rows within the tolerance
     for g in (0, G - 1):
         q1 = q[:, g::G].contiguous()
         out1 = mixture_of_sparse_attention(q1, kc, vc, D ** -0.5, head_start_index=torch.from_numpy(hs).to(dev),
                                            head_valid_length=torch.from_numpy(hv).to(dev))
-        assert torch.equal(out1[:, 0], out[:, 0, g::G])
+        torch.testing.assert_close(out1[:, 0].float(), out[:, 0, g::G].float(), rtol=RTOL, atol=ATOL)
 
 
 def test_grouped_query_70b_shape(dev):
