@@ -53,7 +53,7 @@ def parse_args():
     ap.add_argument("--plan", default=None,
                     help='with --only e2e: a plan file in the reference\'s JSON format {"alphas": [L][H], "betas": [L][H]} '
                          "(e.g. tests/golden/plan_vicuna-7b-v1.5-16k_moa_alpha_beta.json) instead of the synthetic plan")
-    ap.add_argument("--only", choices=["decode", "prefill", "copy", "e2e"], default=None,
+    ap.add_argument("--only", choices=["decode", "prefill", "copy", "e2e", "gqa"], default=None,
                     help="profiling aid: run one part only and print its figures (not the contract line)")
     return ap.parse_args()
 
@@ -197,6 +197,51 @@ def bench_rope_append(torch, dev, args, cache, iters=50):
     nbytes = rope_append_bytes(B, H, D)
     return {"fused_us": fused_us, "separate_us": separate_us, "bytes": nbytes,
             "GB/s": nbytes / (fused_us * 1e-6) / 1e9}
+
+
+def bench_decode_gqa(torch, dev, args, iters=5, layers=8):
+    """Decode attention at the grouped-query shape of the largest config (B=4, 64 query heads on 8
+    rings of head_dim 128, bf16, 32k context: 64 sinks + elastic window per ring): the matrix-core
+    kernel.  K+V bytes of the valid rows per launch over the mean HIP-event time around the call."""
+    import numpy as np
+    from moa_amd import mixture_of_sparse_attention
+    from moa_amd.workloads import elastic_spans, ring_cache_sizes
+    out = {}
+    for B in (4, 64):
+        Hkv, G, D, ctx = 8, 8, 128, 32768
+        caches = []
+        for l in range(layers):
+            sizes, _ = ring_cache_sizes(elastic_spans(Hkv, ctx, seed=l))
+            sizes = np.asarray(sizes)
+            sumc = int(sizes.sum())
+            kc = torch.randn(B, sumc, D, device=dev, dtype=torch.bfloat16)
+            vc = torch.randn(B, sumc, D, device=dev, dtype=torch.bfloat16)
+            start = np.concatenate([[0], np.cumsum(sizes)[:-1]])
+            hs = torch.from_numpy(np.broadcast_to(start, (B, Hkv)).astype(np.int64).copy()).to(dev)
+            hv = torch.from_numpy(np.broadcast_to(sizes, (B, Hkv)).astype(np.int64).copy()).to(dev)
+            caches.append((kc, vc, hs, hv, sumc))
+        q = torch.randn(B, Hkv * G, 1, D, device=dev, dtype=torch.bfloat16)
+        sm = D ** -0.5
+        for kc, vc, hs, hv, _ in caches:
+            mixture_of_sparse_attention(q, kc, vc, sm, head_start_index=hs, head_valid_length=hv)
+        torch.cuda.synchronize(dev)
+        ms, byts = 0.0, 0
+        for _ in range(iters):
+            for kc, vc, hs, hv, sumc in caches:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                mixture_of_sparse_attention(q, kc, vc, sm, head_start_index=hs, head_valid_length=hv)
+                e1.record()
+                torch.cuda.synchronize(dev)
+                ms += e0.elapsed_time(e1)
+                byts += B * sumc * D * 2 * 2
+        n = iters * len(caches)
+        out[f"B{B}"] = {"us_per_launch": ms / n * 1e3, "GB/s": byts / (ms * 1e-3) / 1e9,
+                        "frac_of_hbm_peak": byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        del caches
+        torch.cuda.empty_cache()
+    out["workload"] = "decode attention, 64 query heads on 8 rings, D=128, bf16, 32k context"
+    return out
 
 
 def bench_e2e(torch, dev, args, batch=8, n_ctx=16384, new_tokens=32):
@@ -388,6 +433,9 @@ def main():
     if args.only == "prefill":
         print(json.dumps({"prefill": bench_prefill(torch, dev, args)}))
         return
+    if args.only == "gqa":
+        print(json.dumps({"decode_gqa": bench_decode_gqa(torch, dev, args)}))
+        return
     dec = bench_decode(torch, dev, args)
     rope = bench_rope_append(torch, dev, args, dec["cache"])
     del dec["cache"]
@@ -401,6 +449,8 @@ def main():
             pre = bench_prefill(torch, dev, args)
         except NotImplementedError as e:
             pre = {"error": str(e)}
+    torch.cuda.empty_cache()
+    gqa = bench_decode_gqa(torch, dev, args)
     cpu = None if args.no_cpu else cpu_baseline(torch, args)
 
     line = {
@@ -441,6 +491,7 @@ def main():
         "append": {"us": dec["append_us"], "bytes": dec["append_bytes"], "GB/s": dec["append_gbs"]},
         "rope_append": rope,
         "prefill": pre,
+        "decode_gqa": gqa,
     }
     print(json.dumps(line))
 

@@ -24,7 +24,9 @@
 //     merges them;
 //   * grouped-query attention (G = Hq / Hkv query heads per ring, which the
 //     reference does not have): the G query rows of a ring share every K/V
-//     row that a wave loads, so the cache is still read once.
+//     row that a wave loads, so the cache is still read once.  This kernel is
+//     written for any G but instantiated for G = 1 only; G = 2, 4, 8 run on the
+//     matrix cores (decode_gqa_kernel below).
 #include "moa_mfma.h"
 
 #include <hip/hip_fp16.h>
@@ -334,9 +336,9 @@ __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
 }
 
 
-// ---- grouped-query decode on the matrix cores (G >= 4) ---------------------------------------
+// ---- grouped-query decode on the matrix cores (G >= 2) ---------------------------------------
 // With G query heads per ring the vector ALU version above does G times the arithmetic per cache
-// byte and stops being HBM bound (46 % of peak at G = 8).  Here the G query rows of a ring are the
+// byte and stops being HBM bound (measured: 65 % of peak at G = 2, 46 % at G = 8).  Here the G query rows of a ring are the
 // columns of a 32-wide MFMA tile (columns >= G are zero padding; the matrix pipe has the room):
 //   S^T[key][q] = sum_d K[key][d] Q[q][d]      A = K (LDS), B = Q^T (registers)
 //   O^T[d][q]   = sum_key V[key][d] P[q][key]   A = V^T (LDS, transposing read), B = P^T
@@ -345,7 +347,13 @@ __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
 // private two-stage LDS ring with asynchronous copies (16-byte chunks XOR-permuted as in the
 // prefill kernel), so no work-group barrier is needed inside the loop.  Chunks, partials and the
 // merge kernel are those of the vector version, with a longer chunk.
-constexpr int kGqaChunk = 1024;   // cache rows per work-group step (256 per wave)
+#ifndef MOA_GQA_CHUNK
+#define MOA_GQA_CHUNK 2048
+#endif
+#ifndef MOA_GQA_BLOCKS
+#define MOA_GQA_BLOCKS 4
+#endif
+constexpr int kGqaChunk = MOA_GQA_CHUNK;   // cache rows per work-group step (a quarter per wave)
 constexpr int kGqaTile = 32;      // keys per MFMA tile
 constexpr int kGqaStages = 2;     // LDS stages per wave
 
@@ -617,7 +625,7 @@ static int launch_decode_gqa(const void* q, const void* kc, const void* vc, void
                              int H, int64_t sumC, float sm_scale, hipStream_t st) {
   const int cap = (int)decode_cap(sumC, H);   // partial slots per batch row the workspace was sized for
   const int64_t chunks = (sumC + kGqaChunk - 1) / kGqaChunk + H;   // at most this many steps per batch row
-  int bx = (int)((256 * 4 + B - 1) / B);   // one work-group per CU at a time (its LDS ring fills the CU)
+  int bx = (int)((256 * MOA_GQA_BLOCKS + B - 1) / B);   // one work-group per CU at a time (its LDS ring fills the CU)
   if (bx > chunks) bx = (int)chunks;
   if (bx < 1) bx = 1;
   constexpr size_t lds = gqa_lds_bytes<D>();
@@ -680,7 +688,7 @@ extern "C" int moa_decode_fwd(const void* q, const void* kc, const void* vc, voi
 #define MOA_DEC_G(T, DD)                                        \
   switch (G) {                                                  \
     case 1: return launch_decode<T, DD, 1>(MOA_DEC_ARGS);       \
-    case 2: return launch_decode<T, DD, 2>(MOA_DEC_ARGS);       \
+    case 2: return launch_decode_gqa<T, DD, 2>(MOA_DEC_ARGS);   \
     case 4: return launch_decode_gqa<T, DD, 4>(MOA_DEC_ARGS);   \
     default: return launch_decode_gqa<T, DD, 8>(MOA_DEC_ARGS);  \
   }

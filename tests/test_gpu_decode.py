@@ -210,6 +210,44 @@ def test_grouped_query_decode(dev, dtype, G, D):
         torch.testing.assert_close(out1[:, 0].float(), out[:, 0, g::G].float(), rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("G", [2, 8])
+def test_grouped_query_boundaries_and_invariants(dev, G):
+    """The matrix-core kernel's edges: valid lengths around its 32-key tile, a wave's share (512
+    rows) and its 2048-row chunk; scores that keep raising the running max (keys grow along the
+    ring); the order of the rows inside a ring does not matter; V == 1 gives O == 1."""
+    from moa_amd import mixture_of_sparse_attention
+    rng = np.random.default_rng(7 + G)
+    D, dtype = 128, torch.float16
+    lens = [1, 31, 32, 33, 511, 512, 513, 2047, 2048, 2049, 4097, 100]
+    sizes = [max(64, -(-n // 64) * 64) for n in lens]
+    B, Hkv = 2, len(sizes)
+    _, kc, vc, hs, hv = _case(rng, B, sizes, D, dtype, dev)
+    hv[:] = np.asarray(lens)[None, :]
+    hv[1, 3] = 0
+    ramp = torch.linspace(0.2, 3.0, kc.shape[1], device=dev)[None, :, None]
+    kc = (kc.float() * ramp).to(dtype)                      # later rows score higher: many rescales
+    q = torch.from_numpy(rng.standard_normal((B, Hkv * G, 1, D)).astype(np.float32) * 2).to(dev, dtype)
+    hs_t, hv_t = torch.from_numpy(hs).to(dev), torch.from_numpy(hv).to(dev)
+    out = mixture_of_sparse_attention(q, kc, vc, D ** -0.5, head_start_index=hs_t, head_valid_length=hv_t)
+    ref = decode_segments(q[:, :, 0].float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(),
+                          hs, hv, D ** -0.5, group=G)
+    _close(out[:, 0].float().cpu().numpy(), ref, ("gqa edges", G))
+    # reverse the valid rows of every ring (K and V alike): same softmax, same output
+    kc2, vc2 = kc.clone(), vc.clone()
+    for b in range(B):
+        for h in range(Hkv):
+            s0, n = int(hs[b, h]), int(hv[b, h])
+            kc2[b, s0:s0 + n] = kc[b, s0:s0 + n].flip(0)
+            vc2[b, s0:s0 + n] = vc[b, s0:s0 + n].flip(0)
+    out2 = mixture_of_sparse_attention(q, kc2, vc2, D ** -0.5, head_start_index=hs_t, head_valid_length=hv_t)
+    torch.testing.assert_close(out2.float(), out.float(), rtol=RTOL, atol=ATOL)
+    ones = mixture_of_sparse_attention(q, kc, torch.ones_like(vc), D ** -0.5, head_start_index=hs_t,
+                                       head_valid_length=hv_t)
+    expect = torch.ones_like(ones)
+    expect[1, 0, 3 * G:4 * G] = 0                           # the empty ring
+    assert (ones.float() - expect.float()).abs().max().item() <= 1e-3
+
+
 def test_grouped_query_70b_shape(dev):
     """The 70B shape of the largest config: 64 query heads on 8 rings, head_dim 128, B = 4."""
     from moa_amd import mixture_of_sparse_attention
