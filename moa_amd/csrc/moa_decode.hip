@@ -404,8 +404,8 @@ __global__ __launch_bounds__(kDecThreads) void decode_gqa_kernel(
     const int L = i * 64 + lane;
     const int row = L / CPR, pos = L % CPR;
     crow[i] = row;
-    koff[i] = (uint32_t)((pos ^ ((row / RSH) % CPR)) * 16);
-    voff[i] = (uint32_t)((pos ^ (4 * ((row / RSH) % (CPR / 4)))) * 16);
+    koff[i] = (uint32_t)(row * ROW_B + (pos ^ ((row / RSH) % CPR)) * 16);
+    voff[i] = (uint32_t)(row * ROW_B + (pos ^ (4 * ((row / RSH) % (CPR / 4)))) * 16);
   }
   // operand read addresses inside stage 0 (see the prefill kernel for the layout)
   uint32_t k_ad[KS], v_ad[DT];
@@ -460,11 +460,20 @@ __global__ __launch_bounds__(kDecThreads) void decode_gqa_kernel(
       const char* ksrc = kbase + (int64_t)t * TILE_B;
       const char* vsrc = vbase + (int64_t)t * TILE_B;
       const uint32_t dst = ring0 + (t % kGqaStages) * STAGE_B;
-      const int last = n_rows - 1 - t * kGqaTile;   // >= 0
+      const int last = n_rows - 1 - t * kGqaTile;   // last valid row of the tile, >= 0
+      if (last >= kGqaTile - 1) {
 #pragma unroll
-      for (int i = 0; i < NCP; ++i) async_copy16(ksrc, (uint32_t)(min(crow[i], last) * ROW_B) + koff[i], dst + i * 1024);
+        for (int i = 0; i < NCP; ++i) async_copy16(ksrc, koff[i], dst + i * 1024);
 #pragma unroll
-      for (int i = 0; i < NCP; ++i) async_copy16(vsrc, (uint32_t)(min(crow[i], last) * ROW_B) + voff[i], dst + TILE_B + i * 1024);
+        for (int i = 0; i < NCP; ++i) async_copy16(vsrc, voff[i], dst + TILE_B + i * 1024);
+      } else {
+#pragma unroll
+        for (int i = 0; i < NCP; ++i)
+          async_copy16(ksrc, koff[i] - (uint32_t)(max(crow[i] - last, 0) * ROW_B), dst + i * 1024);
+#pragma unroll
+        for (int i = 0; i < NCP; ++i)
+          async_copy16(vsrc, voff[i] - (uint32_t)(max(crow[i] - last, 0) * ROW_B), dst + TILE_B + i * 1024);
+      }
     };
     if (n_t > 0) issue(0);
     if (n_t > 1) issue(1);
@@ -478,14 +487,16 @@ __global__ __launch_bounds__(kDecThreads) void decode_gqa_kernel(
       const uint32_t so = (uint32_t)((t % kGqaStages) * STAGE_B);
       // ---- S^T = K . Q^T ----
       f32x16 st;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) st[i] = 0.f;
       {
         u32x4 kf[KS];
 #pragma unroll
         for (int s = 0; s < KS; ++s) kf[s] = lds_load16(k_ad[s] + so, 0);
+        f32x16 z;
 #pragma unroll
-        for (int s = 0; s < KS; ++s) st = M::mfma(kf[s], qf[s], st);
+        for (int i = 0; i < 16; ++i) z[i] = 0.f;
+        st = M::mfma(kf[0], qf[0], z);
+#pragma unroll
+        for (int s = 1; s < KS; ++s) st = M::mfma(kf[s], qf[s], st);
       }
       // ---- softmax over the 32 keys (element i of a lane: key 8 (i / 4) + 4 g + i % 4) ----
       const int n_valid = n_rows - t * kGqaTile;
