@@ -319,25 +319,30 @@ def bench_e2e(torch, dev, args, batch=8, n_ctx=16384, new_tokens=32):
             "graph_decode_ms_per_step": graph_s * 1e3, "graph_decode_tokens_per_s": batch / graph_s}
 
 
-def bench_prefill(torch, dev, args):
+def bench_prefill(torch, dev, args, B=4, Hq=32, Hkv=32, N=8192, iters=None):
+    """One sparse prefill layer: the headline shape (B=4, 32 heads, N=8192) by default; the grouped-
+    query shape of the largest config with Hq=64, Hkv=8, N=32768 (spans per kv head)."""
     from moa_amd import mixture_of_sparse_attention
     from moa_amd.workloads import elastic_spans, prefill_work
 
-    B, H, N, D = 4, 32, 8192, 128
+    D = 128
+    H = Hkv
     dtype = torch.bfloat16
     spans = elastic_spans(H, N, seed=0)
     sink = torch.full((H,), 64, dtype=torch.int64, device=dev)
     local = torch.tensor(spans, dtype=torch.int64, device=dev)
     gen = torch.Generator(device=dev).manual_seed(7)
     # the model's projections are [B, N, H, D]; the operator sees them as [B, H, N, D] views
-    q, k, v = (torch.randn(B, N, H, D, generator=gen, device=dev, dtype=dtype).transpose(1, 2) for _ in range(3))
+    q = torch.randn(B, N, Hq, D, generator=gen, device=dev, dtype=dtype).transpose(1, 2)
+    k, v = (torch.randn(B, N, H, D, generator=gen, device=dev, dtype=dtype).transpose(1, 2) for _ in range(2))
     sm = D ** -0.5
     flops, tile_flops, tiles = prefill_work(N, [1] * H, [s // 64 for s in spans], B, D)
-    for _ in range(5):
+    flops, tile_flops = flops * (Hq // Hkv), tile_flops * (Hq // Hkv)
+    for _ in range(5 if iters is None else 2):
         mixture_of_sparse_attention(q, k, v, sm, sink_size=sink, local_size=local)
     torch.cuda.synchronize(dev)
     evs = []
-    for _ in range(args.prefill_iters):
+    for _ in range(args.prefill_iters if iters is None else iters):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         mixture_of_sparse_attention(q, k, v, sm, sink_size=sink, local_size=local)
@@ -347,7 +352,7 @@ def bench_prefill(torch, dev, args):
     ms = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
     med = ms[len(ms) // 2]
     return {
-        "workload": "B=4,H=32,D=128,N=8192,bf16,sink=64,window=elastic(seed 0)",
+        "workload": f"B={B},Hq={Hq},Hkv={Hkv},D=128,N={N},bf16,sink=64,window=elastic(seed 0)",
         "ms_per_layer": med,
         "ms_min": ms[0],
         "flops_live": flops,
@@ -447,6 +452,7 @@ def main():
     if not args.no_prefill:
         try:
             pre = bench_prefill(torch, dev, args)
+            pre["grouped_query_32k"] = bench_prefill(torch, dev, args, B=1, Hq=64, Hkv=8, N=32768, iters=5)
         except NotImplementedError as e:
             pre = {"error": str(e)}
     torch.cuda.empty_cache()
