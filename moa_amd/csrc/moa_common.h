@@ -19,6 +19,23 @@ inline int check_launch(const char* what) {
   return MOA_OK;
 }
 
+// Raises a kernel's dynamic LDS limit.  The attribute belongs to the function on the current device,
+// so it is set once per device; `done` is the caller's per-kernel table.  Two threads racing here both
+// set the same value.
+constexpr int kMaxDevices = 64;
+inline int reserve_lds(const void* kernel, size_t bytes, bool (&done)[kMaxDevices], const char* what) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(MOA_ERR_LAUNCH, "%s: hipGetDevice: %s", what, hipGetErrorString(e));
+  const bool tracked = dev >= 0 && dev < kMaxDevices;
+  if (tracked && done[dev]) return MOA_OK;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e != hipSuccess)
+    return fail(MOA_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS: %s", what, bytes, hipGetErrorString(e));
+  if (tracked) done[dev] = true;
+  return MOA_OK;
+}
+
 inline int elem_bytes(int dtype) {
   switch (dtype) {
     case MOA_DTYPE_F16: return 2;

@@ -640,14 +640,9 @@ static int launch_decode_gqa(const void* q, const void* kc, const void* vc, void
   if (bx > chunks) bx = (int)chunks;
   if (bx < 1) bx = 1;
   constexpr size_t lds = gqa_lds_bytes<D>();
-  static bool attr_set = false;   // per template instance
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_gqa_kernel<T, D, G>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess)
-      return fail(MOA_ERR_LAUNCH, "moa_decode_fwd: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-    attr_set = true;
-  }
+  static bool lds_reserved[kMaxDevices] = {};   // per template instance
+  if (int rc = reserve_lds(reinterpret_cast<const void*>(&decode_gqa_kernel<T, D, G>), lds, lds_reserved, "moa_decode_fwd"))
+    return rc;
   hipLaunchKernelGGL((decode_gqa_kernel<T, D, G>), dim3(bx, B), dim3(kDecThreads), lds, st,
                      (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, (uint16_t*)o,
                      part_acc, part_ml, head_start, head_valid, H, sumC, sm_scale * kLog2e, cap);

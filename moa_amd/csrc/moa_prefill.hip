@@ -485,15 +485,9 @@ static int launch_prefill(const void* q, const void* k, const void* v, void* o, 
   Strides4 sq = {qs[0], qs[1], qs[2]}, sk = {ks[0], ks[1], ks[2]}, sv = {vs[0], vs[1], vs[2]},
            so = {os[0], os[1], os[2]};
   const size_t lds = prefill_lds_bytes<T, D>();
-  static bool attr_set = false;   // per template instance
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_kernel<T, D>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess)
-      return fail(MOA_ERR_LAUNCH, "moa_prefill_fwd: cannot reserve %zu bytes of LDS: %s", lds,
-                  hipGetErrorString(e));
-    attr_set = true;
-  }
+  static bool lds_reserved[kMaxDevices] = {};   // per template instance
+  if (int rc = reserve_lds(reinterpret_cast<const void*>(&prefill_kernel<T, D>), lds, lds_reserved, "moa_prefill_fwd"))
+    return rc;
   hipLaunchKernelGGL((prefill_kernel<T, D>), dim3((unsigned)groups), dim3(kPfThreads), lds, st,
                      (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (uint16_t*)o, sq, sk, sv,
                      so, BH, Hq, Hq / Hkv, N, n_qtiles, sink_blocks, local_blocks, sm_scale * kLog2eF);
