@@ -53,6 +53,9 @@ def parse_args():
     ap.add_argument("--plan", default=None,
                     help='with --only e2e: a plan file in the reference\'s JSON format {"alphas": [L][H], "betas": [L][H]} '
                          "(e.g. tests/golden/plan_vicuna-7b-v1.5-16k_moa_alpha_beta.json) instead of the synthetic plan")
+    ap.add_argument("--shape", choices=["7b", "70b"], default="7b",
+                    help="with --only e2e: 7b = 32 layers, 32 heads, B=8, 16k prompt, fp16; 70b = 80 layers, 64 query "
+                         "heads on 8 kv heads, hidden 8192, B=4, 32k prompt, bf16 (the largest config)")
     ap.add_argument("--only", choices=["decode", "prefill", "copy", "e2e", "gqa"], default=None,
                     help="profiling aid: run one part only and print its figures (not the contract line)")
     return ap.parse_args()
@@ -244,24 +247,29 @@ def bench_decode_gqa(torch, dev, args, iters=5, layers=8):
     return out
 
 
-def bench_e2e(torch, dev, args, batch=8, n_ctx=16384, new_tokens=32):
-    """The attention path of a 7B-shaped decoder end to end (32 layers, hidden 4096, 32 heads of
-    128): q/k/v/o projections (library GEMMs), rotary embedding + cache update, sparse prefill of an
-    n_ctx-token prompt, then new_tokens decode steps.  Norms, MLPs and the LM head are not on the path
-    and are left out.  Random weights; the plan is synthetic (elastic spans) unless --plan names a
-    plan file, whose layer and head counts then set the shape (head dim stays 128)."""
+def bench_e2e(torch, dev, args, new_tokens=32):
+    """The attention path of a decoder end to end: q/k/v/o projections (library GEMMs), rotary
+    embedding + cache update, sparse prefill of the prompt, then new_tokens decode steps.  Norms, MLPs
+    and the LM head are not on the path and are left out.  Shapes: 7b = 32 layers, hidden 4096, 32
+    heads of 128, B=8, 16k prompt, fp16; 70b = 80 layers, hidden 8192, 64 query heads on 8 kv heads,
+    B=4, 32k prompt, bf16.  Random weights; the plan is synthetic (elastic spans per kv head) unless
+    --plan names a plan file, whose layer and head counts then set the shape (head dim stays 128)."""
     from moa_amd.models.llama.modeling_llama import LlamaMixtureAttentionStack
     from moa_amd.workloads import elastic_spans
 
-    L, H, D = args.layers, 32, 128
+    D = 128
+    if args.shape == "70b":
+        L, Hq, H, batch, n_ctx, dtype = 80, 64, 8, 4, 32768, torch.bfloat16
+    else:
+        L, Hq, H, batch, n_ctx, dtype = args.layers, 32, 32, 8, 16384, torch.float16
     plan = None
     if args.plan:
         with open(args.plan) as f:
             plan = json.load(f)
         L, H = len(plan["alphas"]), len(plan["alphas"][0])
-    hidden = H * D
-    dtype = torch.float16
-    model = LlamaMixtureAttentionStack(L, hidden, H, head_dim=D, dtype=dtype, device=dev)
+        Hq = H
+    hidden = Hq * D
+    model = LlamaMixtureAttentionStack(L, hidden, Hq, num_key_value_heads=H, head_dim=D, dtype=dtype, device=dev)
     for p in model.parameters():
         p.data.normal_(0.0, hidden ** -0.5)
     # a plan whose cache sizes are sink (64) + the elastic window at n_ctx
@@ -311,7 +319,8 @@ def bench_e2e(torch, dev, args, batch=8, n_ctx=16384, new_tokens=32):
     torch.cuda.synchronize(dev)
     graph_s = (time.perf_counter() - t0) / new_tokens
     kept = sum(cache.layer_cache_size) / (L * H * (n_ctx + new_tokens))
-    return {"workload": f"attention path of a decoder: L={L}, H={H}, D={D}, B={batch}, prompt {n_ctx}, fp16",
+    return {"workload": f"attention path of a decoder: L={L}, {Hq} query heads on {H} kv heads, D={D}, B={batch}, "
+                        f"prompt {n_ctx}, {str(dtype).split('.')[-1]}",
             "plan": os.path.basename(args.plan) if args.plan else "synthetic elastic spans",
             "kv_kept_fraction": kept,
             "prefill_s": prefill_s, "prefill_tokens_per_s": batch * n_ctx / prefill_s,

@@ -19,14 +19,16 @@ def dev():
     return torch.device("cuda:0")
 
 
-def _make(dev, seed):
+def _make(dev, seed, G):
+    """A cache of 4 rings that holds a 200-token prompt; G query heads per ring."""
     from moa_amd import StaticCircularCache
     B, H, D, S = 2, 4, 128, 200
     cache_size, static = [128, 192, 256, 128], [64] * 4
     cache = StaticCircularCache([cache_size], static_size=[static], batch_size=B, head_dim=D, device=dev,
                                 dtype=torch.float16)
     g = torch.Generator().manual_seed(seed)
-    q, k, v = (torch.randn(B, H, S, D, generator=g).to(dev, torch.float16) for _ in range(3))
+    q = torch.randn(B, H * G, S, D, generator=g).to(dev, torch.float16)
+    k, v = (torch.randn(B, H, S, D, generator=g).to(dev, torch.float16) for _ in range(2))
     cos, sin = rope_cos_sin(torch.arange(S)[None, :], D, dtype=torch.float16)
     cache.rope_update(q, k, v, cos.to(dev), sin.to(dev), 0)
     return cache, (B, H, D, S)
@@ -39,13 +41,15 @@ def _step(cache, q, k, v, cos, sin, D):
                                        head_valid_length=cache.cache_valid_length[0])
 
 
-def test_decode_step_replays_like_eager(dev):
-    cache_g, (B, H, D, S) = _make(dev, 0)      # driven by graph replays
-    cache_e, _ = _make(dev, 0)                 # driven eagerly, same prompt
+@pytest.mark.parametrize("G", [1, 4])   # 1: vector-ALU decode kernel; 4: grouped-query kernel on the matrix cores
+def test_decode_step_replays_like_eager(dev, G):
+    cache_g, (B, H, D, S) = _make(dev, 0, G)   # driven by graph replays
+    cache_e, _ = _make(dev, 0, G)              # driven eagerly, same prompt
     g = torch.Generator().manual_seed(1)
     steps = []
     for t in range(5):
-        q, k, v = (torch.randn(B, H, 1, D, generator=g).to(dev, torch.float16) for _ in range(3))
+        q = torch.randn(B, H * G, 1, D, generator=g).to(dev, torch.float16)
+        k, v = (torch.randn(B, H, 1, D, generator=g).to(dev, torch.float16) for _ in range(2))
         cos, sin = rope_cos_sin(torch.full((1, 1), S + t), D, dtype=torch.float16)
         steps.append((q, k, v, cos.to(dev), sin.to(dev)))
     # static input buffers of the graph; step 0 runs eagerly on a side stream (warm-up: workspaces)
