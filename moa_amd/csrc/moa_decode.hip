@@ -92,27 +92,34 @@ __device__ __forceinline__ uint16_t pack1<BF16>(float x) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Chunk table of one batch row: prefix[h] = number of chunks of heads < h.
-// Built by all threads of the block; returns the row's total chunk count.
+// Built by all threads of the block (one thread per head: kDecThreads >= kMaxHeads): a shuffle
+// scan inside each wave, then the wave totals through LDS.  Returns the row's total chunk count.
 template <int CHUNK>
 __device__ __forceinline__ int build_prefix(const int64_t* __restrict__ valid_row, int H,
                                             int* __restrict__ s_prefix /* [kMaxHeads + 1] */) {
+  __shared__ int s_wave_total[kDecWaves];
   const int tid = threadIdx.x;
-  // kDecThreads >= kMaxHeads: one thread per head, Hillis-Steele scan in LDS
+  const int lane = tid & 63, wave = tid >> 6;
   int n = 0;
   if (tid < H) {
     int64_t len = valid_row[tid];
     if (len < 0) len = 0;
     n = (int)((len + CHUNK - 1) / CHUNK);
   }
-  s_prefix[tid + 1] = n;
+  int incl = n;   // inclusive scan inside the wave
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int up = __shfl_up(incl, off, 64);
+    if (lane >= off) incl += up;
+  }
+  if (lane == 63) s_wave_total[wave] = incl;
+  __syncthreads();
+  int base = 0;
+#pragma unroll
+  for (int w = 0; w < kDecWaves; ++w) base += (w < wave) ? s_wave_total[w] : 0;
+  s_prefix[tid + 1] = base + incl;
   if (tid == 0) s_prefix[0] = 0;
   __syncthreads();
-  for (int off = 1; off < kMaxHeads; off <<= 1) {
-    int add = (tid >= off) ? s_prefix[tid + 1 - off] : 0;
-    __syncthreads();
-    s_prefix[tid + 1] += add;
-    __syncthreads();
-  }
   return s_prefix[H];
 }
 
@@ -297,44 +304,89 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(
 }
 
 // Merge of the per-chunk partials of heads with more than one chunk, and the
-// zero output of empty heads.  One block of D threads per (h, b).
+// zero output of empty heads.  A group of D threads takes one query head at a time: its lanes load
+// the (max, sum) pairs of the chunks side by side, the factors go through LDS, then thread d sums
+// column d of the partial accumulators with several loads in flight.
 template <typename T, int D, int CHUNK, int G>
 __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
     uint16_t* __restrict__ o, const float* __restrict__ part_acc, const float* __restrict__ part_ml,
     const int64_t* __restrict__ head_valid, int H, int cap) {
+  constexpr int GROUPS = kDecThreads / D;
+  constexpr int kFactors = 64;   // chunks whose factors are staged at a time
   __shared__ int s_prefix[kMaxHeads + 1];
+  __shared__ float s_f[GROUPS][kFactors];
+  __shared__ int s_n[GROUPS];
   const int b = blockIdx.y;
   const int tid = threadIdx.x;
   build_prefix<CHUNK>(head_valid + (int64_t)b * H, H, s_prefix);
-  // each group of D threads takes query heads t, t + groups, ... (query head hq reads ring hq / G)
-  constexpr int GROUPS = kDecThreads / D;
   const int grp = tid / D;
   const int d = tid % D;
-  for (int hq = blockIdx.x * GROUPS + grp; hq < H * G; hq += gridDim.x * GROUPS) {
-    const int h = hq / G, g = hq % G;
+  // every group runs the same number of rounds so that the barriers below are uniform
+  const int rounds = (H * G + gridDim.x * GROUPS - 1) / (gridDim.x * GROUPS);
+  for (int r = 0; r < rounds; ++r) {
+    const int hq = (r * gridDim.x + blockIdx.x) * GROUPS + grp;
+    const bool on = hq < H * G;
+    const int h = on ? hq / G : 0, g = on ? hq % G : 0;
     const int w0 = s_prefix[h];
-    const int n = s_prefix[h + 1] - w0;
+    const int n = on ? s_prefix[h + 1] - w0 : 1;
     const int64_t bhq = (int64_t)b * H * G + hq;
-    if (n == 1) continue;  // written by the split kernel
-    if (n == 0) {
-      o[bhq * D + d] = 0;
-      continue;
-    }
     const int64_t slot0 = (int64_t)b * cap + w0;
+    if (on && n == 0) o[bhq * D + d] = 0;
+    // n == 1: written by the split kernel
     float M = -INFINITY;
-    for (int i = 0; i < n; ++i) M = fmaxf(M, part_ml[((slot0 + i) * G + g) * 2]);
+    if (n > 1)
+      for (int i = d; i < n; i += D) M = fmaxf(M, part_ml[((slot0 + i) * G + g) * 2]);
+    // max over the group's lanes (D = 64: one wave; D = 128: two waves, through LDS)
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
+    if (D > 64) {
+      if ((tid & 63) == 0) s_f[grp][(d >> 6)] = M;
+      __syncthreads();
+      M = fmaxf(s_f[grp][0], s_f[grp][1]);
+      __syncthreads();
+    }
     const float m_use = (M == -INFINITY) ? 0.f : M;
     float L = 0.f, a = 0.f;
-    for (int i = 0; i < n; ++i) {
-      const int64_t slot = (slot0 + i) * G + g;
-      const float f = fast_exp2(part_ml[slot * 2] - m_use);
-      L += part_ml[slot * 2 + 1] * f;
-      a += part_acc[slot * D + d] * f;
+    // the groups of a block walk their chunks in lockstep (work-group barriers inside): as many
+    // rounds as the longest of them needs
+    const int n_eff = (n > 1) ? n : 0;
+    if (d == 0) s_n[grp] = n_eff;
+    __syncthreads();
+    int n_loop = 0;
+#pragma unroll
+    for (int k = 0; k < GROUPS; ++k) n_loop = max(n_loop, s_n[k]);
+    for (int i0 = 0; i0 < n_loop; i0 += kFactors) {
+      const int cnt = max(0, min(kFactors, n_eff - i0));
+      if (d < cnt) {
+        const int64_t slot = (slot0 + i0 + d) * G + g;
+        const float f = fast_exp2(part_ml[slot * 2] - m_use);
+        s_f[grp][d] = f;
+        L += part_ml[slot * 2 + 1] * f;
+      }
+      __syncthreads();
+      const float* acc = part_acc + ((slot0 + i0) * G + g) * D + d;
+      int i = 0;
+      for (; i + 4 <= cnt; i += 4) {
+        const float x0 = acc[(int64_t)(i + 0) * G * D], x1 = acc[(int64_t)(i + 1) * G * D];
+        const float x2 = acc[(int64_t)(i + 2) * G * D], x3 = acc[(int64_t)(i + 3) * G * D];
+        a += x0 * s_f[grp][i] + x1 * s_f[grp][i + 1] + x2 * s_f[grp][i + 2] + x3 * s_f[grp][i + 3];
+      }
+      for (; i < cnt; ++i) a += acc[(int64_t)i * G * D] * s_f[grp][i];
+      __syncthreads();
     }
-    o[bhq * D + d] = pack1<T>((L > 0.f) ? a / L : 0.f);
+    // the sum of the group's partial L values
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) L += __shfl_xor(L, off, 64);
+    if (D > 64) {
+      if ((tid & 63) == 0) s_f[grp][(d >> 6)] = L;
+      __syncthreads();
+      L = s_f[grp][0] + s_f[grp][1];
+      __syncthreads();
+    }
+    if (on && n > 1) o[bhq * D + d] = pack1<T>((L > 0.f) ? a / L : 0.f);
+    __syncthreads();   // s_n and s_f are written again in the next round
   }
 }
-
 
 // ---- grouped-query decode on the matrix cores (G >= 2) ---------------------------------------
 // With G query heads per ring the vector ALU version above does G times the arithmetic per cache
