@@ -56,7 +56,8 @@ def parse_args():
     ap.add_argument("--shape", choices=["7b", "70b"], default="7b",
                     help="with --only e2e: 7b = 32 layers, 32 heads, B=8, 16k prompt, fp16; 70b = 80 layers, 64 query "
                          "heads on 8 kv heads, hidden 8192, B=4, 32k prompt, bf16 (the largest config)")
-    ap.add_argument("--only", choices=["decode", "prefill", "copy", "e2e", "gqa"], default=None,
+    ap.add_argument("--new-tokens", type=int, default=64, help="with --only e2e-full: decode steps to time")
+    ap.add_argument("--only", choices=["decode", "prefill", "copy", "e2e", "e2e-full", "gqa"], default=None,
                     help="profiling aid: run one part only and print its figures (not the contract line)")
     return ap.parse_args()
 
@@ -328,6 +329,76 @@ def bench_e2e(torch, dev, args, new_tokens=32):
             "graph_decode_ms_per_step": graph_s * 1e3, "graph_decode_tokens_per_s": batch / graph_s}
 
 
+def bench_e2e_full(torch, dev, args):
+    """The whole decoder of the two end-to-end configs with random bf16 weights: embedding, per
+    layer RMSNorm + attention + RMSNorm + SwiGLU, final norm, LM head, greedy decoding.  7b: 32
+    layers, hidden 4096, 32 heads, FFN 11008, vocab 32000, B=8, 16384-token prompt, spans from alpha
+    in [64, 2048]; 70b: 80 layers, hidden 8192, 64 query heads on 8 kv heads, FFN 28672, vocab 128256,
+    B=4, 32768-token prompt, spans from alpha in [256, 8192]; beta in [0, 0.5] for both.  Only the
+    attention runs in libmoa_hip.so; norms, MLP and LM head are torch (library GEMMs)."""
+    from moa_amd.models.llama.modeling_llama import LlamaMixtureForCausalLM
+    from moa_amd.workloads import elastic_spans
+
+    D, dtype = 128, torch.bfloat16
+    if args.shape == "70b":
+        L, hidden, Hq, H, ffn, vocab, batch, n_ctx, arange = 80, 8192, 64, 8, 28672, 128256, 4, 32768, (256.0, 8192.0)
+    else:
+        L, hidden, Hq, H, ffn, vocab, batch, n_ctx, arange = 32, 4096, 32, 32, 11008, 32000, 8, 16384, (64.0, 2048.0)
+    new_tokens = args.new_tokens
+    model = LlamaMixtureForCausalLM(L, hidden, Hq, H, ffn, vocab, head_dim=D, dtype=dtype, device=dev)
+    for p in model.parameters():
+        if p.dim() > 1:
+            p.data.normal_(0.0, 0.02)
+    plan = {"alphas": [[64 + s for s in elastic_spans(H, n_ctx, seed=l, alpha_range=arange)] for l in range(L)],
+            "betas": [[0.0] * H for _ in range(L)]}
+    model.set_mixture_of_attention(plan, permute_head=True, moa_max_new_token=new_tokens + 8)
+    ids = torch.randint(0, vocab, (batch, n_ctx), generator=torch.Generator().manual_seed(5)).to(dev)
+    times = []
+    for _ in range(2):   # first pass warms up
+        torch.cuda.synchronize(dev)
+        t0 = time.perf_counter()
+        logits, cache = model(ids)
+        torch.cuda.synchronize(dev)
+        times.append(time.perf_counter() - t0)
+    prefill_s = times[-1]
+    tok = logits.argmax(-1, keepdim=True)
+    pos = torch.full((1, 1), n_ctx, device=dev, dtype=torch.int64)
+
+    def step():
+        lg, _ = model(tok, cache, position_ids=pos)
+        tok.copy_(lg.argmax(-1, keepdim=True))
+        pos.add_(1)
+
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    for _ in range(new_tokens):
+        step()
+    torch.cuda.synchronize(dev)
+    dec_s = (time.perf_counter() - t0) / new_tokens
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for _ in range(2):
+        graph.replay()
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    for _ in range(new_tokens):
+        graph.replay()
+    torch.cuda.synchronize(dev)
+    graph_s = (time.perf_counter() - t0) / new_tokens
+    n_param = sum(p.numel() for p in model.parameters())
+    return {"workload": f"whole decoder: L={L}, hidden {hidden}, {Hq} query heads on {H} kv heads, FFN {ffn}, vocab {vocab}, "
+                        f"B={batch}, prompt {n_ctx}, bf16, random weights, greedy",
+            "parameters": n_param,
+            "kv_kept_fraction": sum(cache.layer_cache_size) / (L * H * (n_ctx + new_tokens + 8)),
+            "prefill_s": prefill_s, "prefill_tokens_per_s": batch * n_ctx / prefill_s,
+            "decode_steps_timed": new_tokens,
+            "decode_ms_per_step": dec_s * 1e3, "decode_tokens_per_s": batch / dec_s,
+            "graph_decode_ms_per_step": graph_s * 1e3, "graph_decode_tokens_per_s": batch / graph_s}
+
+
 def bench_prefill(torch, dev, args, B=4, Hq=32, Hkv=32, N=8192, iters=None):
     """One sparse prefill layer: the headline shape (B=4, 32 heads, N=8192) by default; the grouped-
     query shape of the largest config with Hq=64, Hkv=8, N=32768 (spans per kv head)."""
@@ -443,6 +514,9 @@ def main():
         return
     if args.only == "e2e":
         print(json.dumps({"e2e": bench_e2e(torch, dev, args)}))
+        return
+    if args.only == "e2e-full":
+        print(json.dumps({"e2e_full": bench_e2e_full(torch, dev, args)}))
         return
     if args.only == "prefill":
         print(json.dumps({"prefill": bench_prefill(torch, dev, args)}))

@@ -80,6 +80,36 @@ class LlamaMixtureAttention(nn.Module):
         return self.o_proj(attn.reshape(bsz, q_len, self.num_heads * self.head_dim))
 
 
+def install_plan(attention_layers: List["LlamaMixtureAttention"], moa_config: Dict, permute_head: bool) -> Dict:
+    """What ``set_mixture_of_attention`` does to the plan and the projections (reference :373-398):
+    returns the plan as stored on the model (re-ordered like the heads when ``permute_head``)."""
+    alphas = [list(a) for a in moa_config["alphas"]]
+    betas = [list(b) for b in moa_config["betas"]]
+    assert len(alphas) == len(attention_layers) and len(betas) == len(attention_layers)
+    if permute_head:
+        permutations, _ = moa_config_to_permutation({"alphas": alphas, "betas": betas})
+        for layer, perm in zip(attention_layers, permutations):
+            i = layer.layer_idx
+            alphas[i] = [alphas[i][j] for j in perm.tolist()]
+            betas[i] = [betas[i][j] for j in perm.tolist()]
+            hk, g = layer.num_key_value_heads, layer.num_key_value_groups
+            permute_attention_projection(layer.q_proj, perm, hk, g)
+            permute_attention_projection(layer.k_proj, perm, hk)
+            permute_attention_projection(layer.v_proj, perm, hk)
+            permute_output_projection(layer.o_proj, perm, hk, g)
+    return {"alphas": alphas, "betas": betas}
+
+
+def new_cache_for_plan(moa_config: Dict, max_new_token: int, batch_size: int, seq_len: int, head_dim: int,
+                       device, dtype) -> StaticCircularCache:
+    """The cache the reference's model forward builds at the start of a generation
+    (modeling_llama.py:93-112): sizes from the plan at this prompt length."""
+    cfg = moa_config_to_cache_config(moa_config, seq_len, max_new_token=max_new_token, sink_size=64,
+                                     minimum_cache_size=128, split_size=64, verbose=False)
+    return StaticCircularCache(cache_size=cfg["cache_size"], static_size=cfg["static_size"], batch_size=batch_size,
+                               head_dim=head_dim, device=device, dtype=dtype)
+
+
 class LlamaMixtureAttentionStack(nn.Module):
     """The attention path of a decoder: ``num_layers`` attention layers with residual
     connections (norms and MLPs are not on the path and are left out).  Carries what
@@ -106,21 +136,7 @@ class LlamaMixtureAttentionStack(nn.Module):
         clusters heads with equal (alpha, beta): the plan and the q/k/v/o projections of every
         layer are re-ordered consistently (reference :373-398), which leaves the layer's function
         unchanged."""
-        alphas = [list(a) for a in moa_config["alphas"]]
-        betas = [list(b) for b in moa_config["betas"]]
-        assert len(alphas) == len(self.layers) and len(betas) == len(self.layers)
-        if permute_head:
-            permutations, _ = moa_config_to_permutation({"alphas": alphas, "betas": betas})
-            for layer, perm in zip(self.layers, permutations):
-                i = layer.layer_idx
-                alphas[i] = [alphas[i][j] for j in perm.tolist()]
-                betas[i] = [betas[i][j] for j in perm.tolist()]
-                hk, g = layer.num_key_value_heads, layer.num_key_value_groups
-                permute_attention_projection(layer.q_proj, perm, hk, g)
-                permute_attention_projection(layer.k_proj, perm, hk)
-                permute_attention_projection(layer.v_proj, perm, hk)
-                permute_output_projection(layer.o_proj, perm, hk, g)
-        self.moa_config = {"alphas": alphas, "betas": betas}
+        self.moa_config = install_plan(list(self.layers), moa_config, permute_head)
         self.moa_max_new_token = moa_max_new_token
         self.use_moa = True
 
@@ -128,11 +144,8 @@ class LlamaMixtureAttentionStack(nn.Module):
         """The cache the reference's model forward builds at the start of a generation
         (modeling_llama.py:93-112): sizes from the plan at this prompt length."""
         assert self.use_moa, "call set_mixture_of_attention first"
-        cfg = moa_config_to_cache_config(self.moa_config, seq_len, max_new_token=self.moa_max_new_token,
-                                         sink_size=64, minimum_cache_size=128, split_size=64, verbose=False)
-        return StaticCircularCache(cache_size=cfg["cache_size"], static_size=cfg["static_size"],
-                                   batch_size=batch_size, head_dim=self.layers[0].head_dim, device=device,
-                                   dtype=self.dtype)
+        return new_cache_for_plan(self.moa_config, self.moa_max_new_token, batch_size, seq_len,
+                                  self.layers[0].head_dim, device, self.dtype)
 
     @torch.no_grad()
     def forward(self, hidden_states: Tensor, position_ids: Tensor, past_key_value: StaticCircularCache,
@@ -141,3 +154,125 @@ class LlamaMixtureAttentionStack(nn.Module):
         for layer in self.layers:
             hidden_states = hidden_states + layer(hidden_states, (cos, sin), past_key_value, attention_mask)
         return hidden_states
+
+
+class LlamaRMSNorm(nn.Module):
+    """x * rsqrt(mean(x^2) + eps) * weight, the mean in fp32 (plain torch: not on the accelerated path)."""
+
+    def __init__(self, hidden_size: int, eps: float = 1e-5, dtype=torch.float16, device=None):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(hidden_size, dtype=dtype, device=device))
+        self.eps = eps
+
+    def forward(self, x: Tensor) -> Tensor:
+        xf = x.float()
+        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)).to(x.dtype) * self.weight
+
+
+class LlamaMLP(nn.Module):
+    """SwiGLU feed-forward (library GEMMs: not on the accelerated path).  Long prompts go through in
+    slices of ``token_chunk`` tokens so that the intermediate stays small."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, dtype=torch.float16, device=None,
+                 token_chunk: int = 16384):
+        super().__init__()
+        kw = dict(bias=False, dtype=dtype, device=device)
+        self.gate_proj = nn.Linear(hidden_size, intermediate_size, **kw)
+        self.up_proj = nn.Linear(hidden_size, intermediate_size, **kw)
+        self.down_proj = nn.Linear(intermediate_size, hidden_size, **kw)
+        self.token_chunk = token_chunk
+
+    def forward(self, x: Tensor) -> Tensor:
+        flat = x.reshape(-1, x.shape[-1])
+        if flat.shape[0] <= self.token_chunk:
+            return self.down_proj(nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))
+        out = torch.empty_like(flat)
+        for i in range(0, flat.shape[0], self.token_chunk):
+            xs = flat[i:i + self.token_chunk]
+            out[i:i + self.token_chunk] = self.down_proj(nn.functional.silu(self.gate_proj(xs)) * self.up_proj(xs))
+        return out.view_as(x)
+
+
+class LlamaMixtureDecoderLayer(nn.Module):
+    def __init__(self, hidden_size: int, num_heads: int, num_key_value_heads: int, head_dim: int,
+                 intermediate_size: int, layer_idx: int, rms_eps: float, dtype, device):
+        super().__init__()
+        self.input_layernorm = LlamaRMSNorm(hidden_size, rms_eps, dtype, device)
+        self.self_attn = LlamaMixtureAttention(hidden_size, num_heads, num_key_value_heads, head_dim,
+                                               layer_idx=layer_idx, dtype=dtype, device=device)
+        self.post_attention_layernorm = LlamaRMSNorm(hidden_size, rms_eps, dtype, device)
+        self.mlp = LlamaMLP(hidden_size, intermediate_size, dtype, device)
+
+    def forward(self, hidden_states: Tensor, position_embeddings, past_key_value, attention_mask=None) -> Tensor:
+        hidden_states = hidden_states + self.self_attn(self.input_layernorm(hidden_states), position_embeddings,
+                                                       past_key_value, attention_mask)
+        return hidden_states + self.mlp(self.post_attention_layernorm(hidden_states))
+
+
+class LlamaMixtureForCausalLM(nn.Module):
+    """A whole Llama-shaped decoder around the attention path, for end-to-end measurements with
+    random weights: embedding, ``num_layers`` x (RMSNorm, attention, RMSNorm, SwiGLU), final norm,
+    LM head.  Follows the reference's model forward (MoA/models/llama/modeling_llama.py:52-204): the
+    cache is built from the plan at the first call of a generation, positions continue from the
+    cache's length.  Only the attention goes through libmoa_hip.so; the rest is torch."""
+
+    def __init__(self, num_layers: int, hidden_size: int, num_heads: int, num_key_value_heads: int,
+                 intermediate_size: int, vocab_size: int, head_dim: Optional[int] = None,
+                 rope_base: float = 10000.0, rms_eps: float = 1e-5, dtype: torch.dtype = torch.float16, device=None):
+        super().__init__()
+        head_dim = head_dim or hidden_size // num_heads
+        self.embed_tokens = nn.Embedding(vocab_size, hidden_size, dtype=dtype, device=device)
+        self.layers = nn.ModuleList(
+            LlamaMixtureDecoderLayer(hidden_size, num_heads, num_key_value_heads, head_dim, intermediate_size, i,
+                                     rms_eps, dtype, device) for i in range(num_layers))
+        self.norm = LlamaRMSNorm(hidden_size, rms_eps, dtype, device)
+        self.lm_head = nn.Linear(hidden_size, vocab_size, bias=False, dtype=dtype, device=device)
+        self.head_dim = head_dim
+        self.rope_base = rope_base
+        self.dtype = dtype
+        self.use_moa = False
+        self.moa_config: Optional[Dict] = None
+        self.moa_max_new_token = 1024
+        self.eval()
+
+    def set_mixture_of_attention(self, moa_config: Dict, permute_head: bool = False,
+                                 moa_max_new_token: int = 1024) -> None:
+        self.moa_config = install_plan([l.self_attn for l in self.layers], moa_config, permute_head)
+        self.moa_max_new_token = moa_max_new_token
+        self.use_moa = True
+
+    @torch.no_grad()
+    def forward(self, input_ids: Tensor, past_key_values: Optional[StaticCircularCache] = None,
+                attention_mask: Optional[Tensor] = None, position_ids: Optional[Tensor] = None
+                ) -> Tuple[Tensor, StaticCircularCache]:
+        """input_ids ``[batch, q_len]``.  Returns the logits of the last position ``[batch, vocab]`` and
+        the cache (created here when none is passed).  ``position_ids`` ``[1 or batch, q_len]`` default
+        to the positions after the cache's length; a caller that replays a captured decode step passes
+        a device tensor that it advances itself."""
+        assert self.use_moa, "call set_mixture_of_attention first"
+        bsz, q_len = input_ids.shape
+        if past_key_values is None:
+            past_key_values = new_cache_for_plan(self.moa_config, self.moa_max_new_token, bsz, q_len,
+                                                 self.head_dim, input_ids.device, self.dtype)
+        if position_ids is None:
+            past = past_key_values.get_seq_length()
+            position_ids = torch.arange(past, past + q_len, device=input_ids.device)[None, :]
+        if attention_mask is not None and not (attention_mask == 0).any():
+            attention_mask = None    # as the reference: a mask without padding is no mask (:119-121)
+        cos_sin = rotary_cos_sin(position_ids, self.head_dim, self.dtype, self.rope_base)
+        hidden_states = self.embed_tokens(input_ids)
+        for layer in self.layers:
+            hidden_states = layer(hidden_states, cos_sin, past_key_values, attention_mask)
+        logits = self.lm_head(self.norm(hidden_states[:, -1, :]))
+        return logits, past_key_values
+
+    @torch.no_grad()
+    def generate_greedy(self, input_ids: Tensor, max_new_tokens: int) -> Tensor:
+        """Prompt, then ``max_new_tokens`` greedy steps.  Returns the new token ids ``[batch, max_new_tokens]``."""
+        logits, cache = self.forward(input_ids)
+        out = []
+        for _ in range(max_new_tokens):
+            nxt = logits.argmax(-1, keepdim=True)
+            out.append(nxt)
+            logits, cache = self.forward(nxt, cache)
+        return torch.cat(out, dim=1)
