@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L]
 
-Headline workload (BASELINE.json configs[2], the one the metric is quoted on):
+Headline workload (the configuration the metric is quoted on):
 decode step + cache append at the 7B shape -- batch 64, 32 heads, head_dim 128,
 fp16, logical context 16384, every (layer, head) with its own ring of
 64 sinks + elastic window.  One "step" generates one token for the whole batch
@@ -14,7 +14,7 @@ projections/MLP of a full decoder are not part of this path and not run.
 value = batch * steps / wall seconds (whole job, inputs resident in HBM).
 
 Also measured, outside the timed region, and reported in the same JSON line:
-  * sparse prefill (configs[1]): B=4, H=32, D=128, N=8192, bf16 -> ms/layer,
+  * sparse prefill: B=4, H=32, D=128, N=8192, bf16 -> ms/layer,
     TFLOP/s on live (unmasked) work, fraction of the dense bf16 MFMA peak;
   * the append kernel alone (us, GB/s);
   * cpu_baseline: the CPU oracle's restatement of the reference's dense

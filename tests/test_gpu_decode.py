@@ -2,8 +2,8 @@
 libmoa_hip.so) against the fp64 CPU oracle.
 
 Tolerance (fp16/bf16 inputs, fp32 softmax, output rounded to the input dtype):
-|out - oracle| <= 2e-3 + 1e-2 * |oracle|, the bound BASELINE states for this
-path, applied the way the reference's tests apply theirs (assert_close)."""
+|out - oracle| <= 2e-3 + 1e-2 * |oracle|, the bound this path is specified with
+(max-abs 2e-3, relative 1e-2), applied the way the reference's tests apply theirs (assert_close)."""
 import numpy as np
 import pytest
 import torch
