@@ -91,9 +91,9 @@ size_t moa_decode_workspace_bytes(int B, int Hq, int Hkv, int D, int64_t sumC);
  * the packed cache; the workspace is sized for that.
  * Query head h reads ring h / (Hq/Hkv): grouped-query attention, which the
  * reference does not have (its caller asserts one kv group,
- * MoA/models/llama/modeling_llama.py:220-224), with Hq/Hkv in {1,2,4,8}.
+ * MoA/models/llama/modeling_llama.py:220-224), with Hq/Hkv in 1..8.
  * With one query head per ring the kernel works on the vector ALU in fp32;
- * with 2, 4 or 8 it works on the matrix cores and rounds the softmax weights
+ * with 2 to 8 it works on the matrix cores and rounds the softmax weights
  * to the input type before multiplying with V (like the prefill kernel).
  * D in {64,128}, f16/bf16, at most 256 kv heads.
  */

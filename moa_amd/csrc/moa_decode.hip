@@ -307,10 +307,10 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(
 // zero output of empty heads.  A group of D threads takes one query head at a time: its lanes load
 // the (max, sum) pairs of the chunks side by side, the factors go through LDS, then thread d sums
 // column d of the partial accumulators with several loads in flight.
-template <typename T, int D, int CHUNK, int G>
+template <typename T, int D, int CHUNK>
 __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
     uint16_t* __restrict__ o, const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-    const int64_t* __restrict__ head_valid, int H, int cap) {
+    const int64_t* __restrict__ head_valid, int H, int G /* query heads per ring */, int cap) {
   constexpr int GROUPS = kDecThreads / D;
   constexpr int kFactors = 64;   // chunks whose factors are staged at a time
   __shared__ int s_prefix[kMaxHeads + 1];
@@ -407,6 +407,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
 #endif
 constexpr int kGqaChunk = MOA_GQA_CHUNK;   // cache rows per work-group step (a quarter per wave)
 constexpr int kGqaTile = 32;      // keys per MFMA tile
+constexpr int kGqaMaxG = 8;       // query heads per ring the per-wave result buffers are sized for
 constexpr int kGqaStages = 2;     // LDS stages per wave
 
 template <typename T> struct MfmaElem;
@@ -416,12 +417,12 @@ template <> struct MfmaElem<BF16> { typedef PBF16 type; };
 template <int D>
 constexpr size_t gqa_lds_bytes() { return (size_t)kDecWaves * kGqaStages * 2 * kGqaTile * D * 2; }
 
-template <typename T, int D, int G>
+template <typename T, int D>
 __global__ __launch_bounds__(kDecThreads) void decode_gqa_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     uint16_t* __restrict__ o, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const int64_t* __restrict__ head_start, const int64_t* __restrict__ head_valid, int H,
-    int64_t sumC, float scale_log2, int cap) {
+    int G /* query heads per ring, <= kGqaMaxG */, int64_t sumC, float scale_log2, int cap) {
   typedef typename MfmaElem<T>::type M;
   constexpr int KS = D / 16;                    // MFMA k-steps of Q.K^T
   constexpr int DT = D / 32;                    // 32-wide d tiles of the output
@@ -436,9 +437,9 @@ __global__ __launch_bounds__(kDecThreads) void decode_gqa_kernel(
 
   extern __shared__ __attribute__((aligned(1024))) char s_mem[];
   __shared__ int s_prefix[kMaxHeads + 1];
-  __shared__ float s_acc[kDecWaves][G][D];
-  __shared__ float s_m[kDecWaves][G];
-  __shared__ float s_l[kDecWaves][G];
+  __shared__ float s_acc[kDecWaves][kGqaMaxG][D];
+  __shared__ float s_m[kDecWaves][kGqaMaxG];
+  __shared__ float s_l[kDecWaves][kGqaMaxG];
 
   const int b = blockIdx.y;
   const int tid = threadIdx.x;
@@ -615,7 +616,6 @@ __global__ __launch_bounds__(kDecThreads) void decode_gqa_kernel(
 
     // ---- combine the waves; thread d owns output column d of every query head of the ring ----
     if (tid < D) {
-#pragma unroll
       for (int gq = 0; gq < G; ++gq) {
         float Mx = s_m[0][gq];
 #pragma unroll
@@ -676,16 +676,16 @@ static int launch_decode(const void* q, const void* kc, const void* vc, void* o,
   if (rc) return rc;
   constexpr int GROUPS = kDecThreads / D;
   int mx = (H * G + GROUPS - 1) / GROUPS;
-  hipLaunchKernelGGL((decode_merge_kernel<T, D, kChunk, G>), dim3(mx, B), dim3(kDecThreads), 0, st,
-                     (uint16_t*)o, part_acc, part_ml, head_valid, H, cap);
+  hipLaunchKernelGGL((decode_merge_kernel<T, D, kChunk>), dim3(mx, B), dim3(kDecThreads), 0, st,
+                     (uint16_t*)o, part_acc, part_ml, head_valid, H, G, cap);
   return check_launch("moa_decode_fwd(merge)");
 }
 
 
-template <typename T, int D, int G>
+template <typename T, int D>
 static int launch_decode_gqa(const void* q, const void* kc, const void* vc, void* o, float* part_acc,
                              float* part_ml, const int64_t* head_start, const int64_t* head_valid, int B,
-                             int H, int64_t sumC, float sm_scale, hipStream_t st) {
+                             int H, int G, int64_t sumC, float sm_scale, hipStream_t st) {
   const int cap = (int)decode_cap(sumC, H);   // partial slots per batch row the workspace was sized for
   const int64_t chunks = (sumC + kGqaChunk - 1) / kGqaChunk + H;   // at most this many steps per batch row
   int bx = (int)((256 * MOA_GQA_BLOCKS + B - 1) / B);   // one work-group per CU at a time (its LDS ring fills the CU)
@@ -693,17 +693,17 @@ static int launch_decode_gqa(const void* q, const void* kc, const void* vc, void
   if (bx < 1) bx = 1;
   constexpr size_t lds = gqa_lds_bytes<D>();
   static bool lds_reserved[kMaxDevices] = {};   // per template instance
-  if (int rc = reserve_lds(reinterpret_cast<const void*>(&decode_gqa_kernel<T, D, G>), lds, lds_reserved, "moa_decode_fwd"))
+  if (int rc = reserve_lds(reinterpret_cast<const void*>(&decode_gqa_kernel<T, D>), lds, lds_reserved, "moa_decode_fwd"))
     return rc;
-  hipLaunchKernelGGL((decode_gqa_kernel<T, D, G>), dim3(bx, B), dim3(kDecThreads), lds, st,
+  hipLaunchKernelGGL((decode_gqa_kernel<T, D>), dim3(bx, B), dim3(kDecThreads), lds, st,
                      (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, (uint16_t*)o,
-                     part_acc, part_ml, head_start, head_valid, H, sumC, sm_scale * kLog2e, cap);
+                     part_acc, part_ml, head_start, head_valid, H, G, sumC, sm_scale * kLog2e, cap);
   int rc = check_launch("moa_decode_fwd(grouped split)");
   if (rc) return rc;
   constexpr int GROUPS = kDecThreads / D;
   int mx = (H * G + GROUPS - 1) / GROUPS;
-  hipLaunchKernelGGL((decode_merge_kernel<T, D, kGqaChunk, G>), dim3(mx, B), dim3(kDecThreads), 0, st,
-                     (uint16_t*)o, part_acc, part_ml, head_valid, H, cap);
+  hipLaunchKernelGGL((decode_merge_kernel<T, D, kGqaChunk>), dim3(mx, B), dim3(kDecThreads), 0, st,
+                     (uint16_t*)o, part_acc, part_ml, head_valid, H, G, cap);
   return check_launch("moa_decode_fwd(merge)");
 }
 
@@ -727,8 +727,8 @@ extern "C" int moa_decode_fwd(const void* q, const void* kc, const void* vc, voi
   if (B > 65535) return fail(MOA_ERR_UNSUPPORTED, "moa_decode_fwd: B <= 65535");
   if (Hq % Hkv != 0) return fail(MOA_ERR_ARG, "moa_decode_fwd: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
   const int G = Hq / Hkv;
-  if (G != 1 && G != 2 && G != 4 && G != 8)
-    return fail(MOA_ERR_UNSUPPORTED, "moa_decode_fwd: %d query heads per kv head (1, 2, 4 or 8)", G);
+  if (G > kGqaMaxG)
+    return fail(MOA_ERR_UNSUPPORTED, "moa_decode_fwd: %d query heads per kv head (at most %d)", G, kGqaMaxG);
   if (Hkv > kMaxHeads) return fail(MOA_ERR_UNSUPPORTED, "moa_decode_fwd: at most %d kv heads", kMaxHeads);
   if (D != 64 && D != 128) return fail(MOA_ERR_UNSUPPORTED, "moa_decode_fwd: head_dim %d (64 or 128)", D);
   if (dtype != MOA_DTYPE_F16 && dtype != MOA_DTYPE_BF16)
@@ -742,20 +742,15 @@ extern "C" int moa_decode_fwd(const void* q, const void* kc, const void* vc, voi
   float* part_acc = reinterpret_cast<float*>(workspace);
   float* part_ml = part_acc + slots * (size_t)D;
   hipStream_t st = (hipStream_t)stream;
-#define MOA_DEC_ARGS q, kc, vc, o, part_acc, part_ml, head_start, head_valid_len, B, Hkv, sumC, sm_scale, st
-#define MOA_DEC_G(T, DD)                                        \
-  switch (G) {                                                  \
-    case 1: return launch_decode<T, DD, 1>(MOA_DEC_ARGS);       \
-    case 2: return launch_decode_gqa<T, DD, 2>(MOA_DEC_ARGS);   \
-    case 4: return launch_decode_gqa<T, DD, 4>(MOA_DEC_ARGS);   \
-    default: return launch_decode_gqa<T, DD, 8>(MOA_DEC_ARGS);  \
-  }
+#define MOA_DEC_ARGS q, kc, vc, o, part_acc, part_ml, head_start, head_valid_len, B, Hkv
+#define MOA_DEC_TAIL sumC, sm_scale, st
+  // one query head per ring: vector ALU kernel; more: matrix-core kernel
   if (dtype == MOA_DTYPE_F16) {
-    if (D == 128) { MOA_DEC_G(F16, 128) }
-    MOA_DEC_G(F16, 64)
+    if (D == 128) return G == 1 ? launch_decode<F16, 128, 1>(MOA_DEC_ARGS, MOA_DEC_TAIL) : launch_decode_gqa<F16, 128>(MOA_DEC_ARGS, G, MOA_DEC_TAIL);
+    return G == 1 ? launch_decode<F16, 64, 1>(MOA_DEC_ARGS, MOA_DEC_TAIL) : launch_decode_gqa<F16, 64>(MOA_DEC_ARGS, G, MOA_DEC_TAIL);
   }
-  if (D == 128) { MOA_DEC_G(BF16, 128) }
-  MOA_DEC_G(BF16, 64)
-#undef MOA_DEC_G
+  if (D == 128) return G == 1 ? launch_decode<BF16, 128, 1>(MOA_DEC_ARGS, MOA_DEC_TAIL) : launch_decode_gqa<BF16, 128>(MOA_DEC_ARGS, G, MOA_DEC_TAIL);
+  return G == 1 ? launch_decode<BF16, 64, 1>(MOA_DEC_ARGS, MOA_DEC_TAIL) : launch_decode_gqa<BF16, 64>(MOA_DEC_ARGS, G, MOA_DEC_TAIL);
+#undef MOA_DEC_TAIL
 #undef MOA_DEC_ARGS
 }

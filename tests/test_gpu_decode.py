@@ -181,7 +181,7 @@ def test_decode_config_scale(dev):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("G", [2, 4, 8])
+@pytest.mark.parametrize("G", [2, 3, 4, 5, 7, 8])
 @pytest.mark.parametrize("D", [128, 64])
 def test_grouped_query_decode(dev, dtype, G, D):
     """G query heads per ring (not in the reference, whose caller asserts one kv group,
@@ -293,9 +293,9 @@ def test_errors(dev):
     k96 = torch.zeros(1, 256, 96, dtype=torch.float16, device=dev)
     with pytest.raises(NotImplementedError):  # head_dim 96 is not covered
         mixture_of_sparse_attention(q96, k96, k96, 1.0, head_start_index=hs, head_valid_length=hv)
-    q6 = torch.zeros(1, 6, 1, 128, dtype=torch.float16, device=dev)
-    with pytest.raises(NotImplementedError):  # 3 query heads per ring is not covered
-        mixture_of_sparse_attention(q6, k.half(), k.half(), 1.0, head_start_index=hs, head_valid_length=hv)
+    q18 = torch.zeros(1, 18, 1, 128, dtype=torch.float16, device=dev)
+    with pytest.raises(NotImplementedError):  # 9 query heads per ring: more than the kernel's 8
+        mixture_of_sparse_attention(q18, k.half(), k.half(), 1.0, head_start_index=hs, head_valid_length=hv)
     q3 = torch.zeros(1, 3, 1, 128, dtype=torch.float16, device=dev)
     with pytest.raises(AssertionError):       # 3 query heads do not divide over 2 rings
         mixture_of_sparse_attention(q3, k.half(), k.half(), 1.0, head_start_index=hs, head_valid_length=hv)
