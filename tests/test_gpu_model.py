@@ -39,9 +39,9 @@ def _plan(layers, kv_heads, alpha):
     return {"alphas": [[alpha] * kv_heads for _ in range(layers)], "betas": [[0.0] * kv_heads for _ in range(layers)]}
 
 
-@pytest.mark.parametrize("kv_heads", [4, 2, 1])
-def test_incremental_decoding_matches_one_shot_prompt(dev, kv_heads):
-    m = _model(dev, heads=4, kv_heads=kv_heads)
+@pytest.mark.parametrize("heads,kv_heads", [(4, 4), (4, 2), (4, 1), (6, 2)])
+def test_incremental_decoding_matches_one_shot_prompt(dev, heads, kv_heads):
+    m = _model(dev, heads=heads, kv_heads=kv_heads)
     m.set_mixture_of_attention(_plan(2, kv_heads, 4096.0), moa_max_new_token=64)   # rings hold everything
     g = torch.Generator().manual_seed(1)
     ids = torch.randint(0, 1000, (2, 137), generator=g).to(dev)
