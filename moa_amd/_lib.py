@@ -122,8 +122,13 @@ def dtype_code(torch_dtype) -> int:
 
 
 def current_stream_ptr(device) -> int:
+    """The raw HIP stream torch is currently using on ``device`` (through torch's internal accessor
+    when it exists: the public ``torch.cuda.current_stream`` costs several microseconds per call)."""
     import torch
 
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if raw is not None:
+        return raw(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
 
 

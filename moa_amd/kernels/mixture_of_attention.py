@@ -24,10 +24,10 @@ BLOCK_N = 64
 _workspaces: Dict[Tuple[int, int, str], Tensor] = {}
 
 
-def _workspace(device: torch.device, nbytes: int, tag: str) -> Tensor:
+def _workspace(device: torch.device, nbytes: int, tag: str, stream: int) -> Tensor:
     """A per-(device, stream) scratch buffer that only ever grows, so steady
     state calls allocate nothing."""
-    key = (device.index or 0, torch.cuda.current_stream(device).cuda_stream, tag)
+    key = (device.index or 0, stream, tag)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
@@ -138,10 +138,11 @@ def moa_decode(
     o = torch.empty((B, 1, Hq, D), dtype=q.dtype, device=dev)
     lib = _lib.load()
     need = lib.moa_decode_workspace_bytes(B, Hq, Hkv, D, sumC)
-    ws = _workspace(dev, need, "decode")
+    stream = _lib.current_stream_ptr(dev)
+    ws = _workspace(dev, need, "decode", stream)
     rc = lib.moa_decode_fwd(q3.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ws.data_ptr(),
                             ws.numel(), hs.data_ptr(), hv.data_ptr(), B, Hq, Hkv, D, sumC,
-                            float(sm_scale), _lib.dtype_code(q.dtype), _lib.current_stream_ptr(dev))
+                            float(sm_scale), _lib.dtype_code(q.dtype), stream)
     _lib.check(rc)
     return o
 
