@@ -99,10 +99,10 @@ struct DecInt {
 // Chunk table of one batch row: prefix[h] = number of chunks of heads < h.
 // Built by all threads of the block (one thread per head: kDecThreads >= kMaxHeads): a shuffle
 // scan inside each wave, then the wave totals through LDS.  Returns the row's total chunk count.
-template <int CHUNK>
+template <int CHUNK, int NWAVES = kDecWaves>
 __device__ __forceinline__ int build_prefix(const int64_t* __restrict__ valid_row, int H,
                                             int* __restrict__ s_prefix /* [kMaxHeads + 1] */) {
-  __shared__ int s_wave_total[kDecWaves];
+  __shared__ int s_wave_total[NWAVES];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   int n = 0;
@@ -121,8 +121,8 @@ __device__ __forceinline__ int build_prefix(const int64_t* __restrict__ valid_ro
   __syncthreads();
   int base = 0;
 #pragma unroll
-  for (int w = 0; w < kDecWaves; ++w) base += (w < wave) ? s_wave_total[w] : 0;
-  s_prefix[tid + 1] = base + incl;
+  for (int w = 0; w < NWAVES; ++w) base += (w < wave) ? s_wave_total[w] : 0;
+  if (tid < kMaxHeads) s_prefix[tid + 1] = base + incl;
   if (tid == 0) s_prefix[0] = 0;
   __syncthreads();
   return s_prefix[H];
@@ -442,17 +442,22 @@ __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
 constexpr int kGqaChunk = MOA_GQA_CHUNK;   // cache rows per work-group step (a quarter per wave)
 constexpr int kGqaTile = 32;      // keys per MFMA tile
 constexpr int kGqaMaxG = 8;       // query heads per ring the per-wave result buffers are sized for
-constexpr int kGqaStages = 2;     // LDS stages per wave
+#ifndef MOA_GQA_WAVES
+#define MOA_GQA_WAVES 4
+#endif
+constexpr int kGqaWaves = MOA_GQA_WAVES;          // waves per work-group
+constexpr int kGqaThreads = 64 * kGqaWaves;
+constexpr int kGqaStages = 8 / kGqaWaves;         // LDS stages per wave (8 stages of 16 KiB at D = 128 in all)
 
 template <typename T> struct MfmaElem;
 template <> struct MfmaElem<F16> { typedef PF16 type; };
 template <> struct MfmaElem<BF16> { typedef PBF16 type; };
 
 template <int D>
-constexpr size_t gqa_lds_bytes() { return (size_t)kDecWaves * kGqaStages * 2 * kGqaTile * D * 2; }
+constexpr size_t gqa_lds_bytes() { return (size_t)kGqaWaves * kGqaStages * 2 * kGqaTile * D * 2; }
 
 template <typename T, int D>
-__global__ __launch_bounds__(kDecThreads) void decode_gqa_kernel(
+__global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     uint16_t* __restrict__ o, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const int64_t* __restrict__ head_start, const int64_t* __restrict__ head_valid, int H,
@@ -466,14 +471,16 @@ __global__ __launch_bounds__(kDecThreads) void decode_gqa_kernel(
   constexpr int TILE_B = kGqaTile * ROW_B;      // bytes of one K or V tile
   constexpr int NCP = TILE_B / 1024;            // async copies per tile and tensor
   constexpr int STAGE_B = 2 * TILE_B;           // K tile, then V tile
-  constexpr int WCHUNK = kGqaChunk / kDecWaves;
+  constexpr int WCHUNK = kGqaChunk / kGqaWaves;
   constexpr float kRescaleStep = 8.f;
 
   extern __shared__ __attribute__((aligned(1024))) char s_mem[];
   __shared__ int s_prefix[kMaxHeads + 1];
-  __shared__ float s_acc[kDecWaves][kGqaMaxG][D];
-  __shared__ float s_m[kDecWaves][kGqaMaxG];
-  __shared__ float s_l[kDecWaves][kGqaMaxG];
+  // the per-wave results (m, l, O[d] per query head) go into the first 4.5 KiB of the wave's own ring
+  // once its loop is over
+  __shared__ float s_m[kGqaWaves][kGqaMaxG];
+  __shared__ float s_l[kGqaWaves][kGqaMaxG];
+  static_assert(kGqaMaxG * D * 4 <= kGqaStages * STAGE_B, "the result buffer fits the wave's ring");
 
   const int b = blockIdx.y;
   const int tid = threadIdx.x;
@@ -508,7 +515,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_gqa_kernel(
     for (int dt = 0; dt < DT; ++dt) v_ad[dt] = ring0 + TILE_B + (v_rd ^ (uint32_t)(64 * dt));
   }
 
-  const int total = min(build_prefix<kGqaChunk>(head_valid + (int64_t)b * H, H, s_prefix), cap);
+  const int total = min(build_prefix<kGqaChunk, kGqaWaves>(head_valid + (int64_t)b * H, H, s_prefix), cap);
 
   for (int w = blockIdx.x; w < total; w += gridDim.x) {
     const int h = find_head(s_prefix, H, w);
@@ -563,14 +570,14 @@ __global__ __launch_bounds__(kDecThreads) void decode_gqa_kernel(
       }
     };
     if (n_t > 0) issue(0);
-    if (n_t > 1) issue(1);
+    if (kGqaStages > 1 && n_t > 1) issue(1);
     // the Q loads are older than every copy: pin their arrival here
-    if (n_t > 1) wait_vm(4 * NCP); else if (n_t > 0) wait_vm(2 * NCP);
+    if (kGqaStages > 1 && n_t > 1) wait_vm(4 * NCP); else if (n_t > 0) wait_vm(2 * NCP);
 #pragma unroll
     for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[s]));
 
     for (int t = 0; t < n_t; ++t) {
-      if (t + 1 < n_t) wait_vm(2 * NCP); else wait_vm(0);     // tile t has landed; tile t+1 may be in flight
+      if (kGqaStages > 1 && t + 1 < n_t) wait_vm(2 * NCP); else wait_vm(0);   // tile t has landed; tile t+1 may be in flight
       const uint32_t so = (uint32_t)((t % kGqaStages) * STAGE_B);
       // ---- S^T = K . Q^T ----
       f32x16 st;
@@ -635,11 +642,12 @@ __global__ __launch_bounds__(kDecThreads) void decode_gqa_kernel(
     // ---- the wave's result per query head: (m, l, O[d]) ----
     {
       const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+      float* s_acc_w = reinterpret_cast<float*>(s_mem + wave * (kGqaStages * STAGE_B));
       if (mcol < G) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) s_acc[wave][mcol][32 * dt + 8 * (i >> 2) + 4 * g + (i & 3)] = oacc[dt][i];
+          for (int i = 0; i < 16; ++i) s_acc_w[mcol * D + 32 * dt + 8 * (i >> 2) + 4 * g + (i & 3)] = oacc[dt][i];
         if (g == 0) {
           s_m[wave][mcol] = m_run;
           s_l[wave][mcol] = l_tot;
@@ -653,14 +661,14 @@ __global__ __launch_bounds__(kDecThreads) void decode_gqa_kernel(
       for (int gq = 0; gq < G; ++gq) {
         float Mx = s_m[0][gq];
 #pragma unroll
-        for (int i = 1; i < kDecWaves; ++i) Mx = fmaxf(Mx, s_m[i][gq]);
+        for (int i = 1; i < kGqaWaves; ++i) Mx = fmaxf(Mx, s_m[i][gq]);
         const float m_use = (Mx == -INFINITY) ? 0.f : Mx;
         float L = 0.f, a = 0.f;
 #pragma unroll
-        for (int i = 0; i < kDecWaves; ++i) {
+        for (int i = 0; i < kGqaWaves; ++i) {
           const float f = fast_exp2(s_m[i][gq] - m_use);
           L += s_l[i][gq] * f;
-          a += s_acc[i][gq][tid] * f;
+          a += reinterpret_cast<const float*>(s_mem + i * (kGqaStages * STAGE_B))[gq * D + tid] * f;
         }
         if (n_chunks == 1) {
           o[(bh * G + gq) * D + tid] = pack1<T>((L > 0.f) ? a / L : 0.f);
@@ -738,7 +746,7 @@ static int launch_decode_gqa(const void* q, const void* kc, const void* vc, void
   static bool lds_reserved[kMaxDevices] = {};   // per template instance
   if (int rc = reserve_lds(reinterpret_cast<const void*>(&decode_gqa_kernel<T, D>), lds, lds_reserved, "moa_decode_fwd"))
     return rc;
-  hipLaunchKernelGGL((decode_gqa_kernel<T, D>), dim3(bx, B), dim3(kDecThreads), lds, st,
+  hipLaunchKernelGGL((decode_gqa_kernel<T, D>), dim3(bx, B), dim3(kGqaThreads), lds, st,
                      (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, (uint16_t*)o,
                      part_acc, part_ml, head_start, head_valid, H, G, sumC, sm_scale * kLog2e, cap);
   int rc = check_launch("moa_decode_fwd(grouped split)");
