@@ -99,6 +99,28 @@ def test_small_against_oracle(dev, dtype, D, N):
     _close(out, ref, (dtype, D, N))
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_plans_against_oracle(dev, seed):
+    """Random lengths (ragged and long enough for several 256-row query tiles), random sink and band
+    block counts per head incl. 0 and more than there are blocks: the tile schedule (sinks, rotated
+    band, wrap, repeated last tile) against the dense masked oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    D = int(rng.choice([64, 128]))
+    dtype = [torch.float16, torch.bfloat16][seed % 2]
+    N = int(rng.integers(65, 1800))
+    nb = -(-N // 64)
+    H = int(rng.integers(1, 7))
+    ns = [int(x) for x in rng.integers(0, min(nb, 6) + 2, size=H)]
+    nl = [int(x) for x in rng.integers(0, nb + 3, size=H)]
+    if seed % 5 == 0:
+        nl = [int(x) for x in rng.integers(0, 4, size=H)]      # narrow bands: many dead tiles per query tile
+    q, k, v = _qkv(1 + seed % 2, H, N, D, dtype, dev, seed=seed)
+    sm = D ** -0.5
+    out = _run(q, k, v, sm, ns, nl, dev)
+    ref = prefill_masked_dense(q, k, v, sm, ns, nl)
+    _close(out, ref, (seed, N, D, ns, nl))
+
+
 def test_dead_rows_are_zero(dev):
     """ns = nl = 0 sees nothing; nl = 0 with sinks sees only sink blocks."""
     q, k, v = _qkv(1, 2, 256, 128, torch.float16, dev, seed=3)
