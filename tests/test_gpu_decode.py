@@ -261,6 +261,38 @@ def test_grouped_query_boundaries_and_invariants(dev, G):
     assert (ones.float() - expect.float()).abs().max().item() <= 1e-3
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_random_layouts(dev, seed):
+    """Segments anywhere in the packed row (gaps between them, not in head order), random valid
+    lengths incl. 0, 1..8 query heads per ring, both head dims and dtypes."""
+    from moa_amd import mixture_of_sparse_attention
+    rng = np.random.default_rng(500 + seed)
+    D = int(rng.choice([64, 128]))
+    dtype = [torch.float16, torch.bfloat16][seed % 2]
+    G = int(rng.integers(1, 9))
+    B, Hkv = int(rng.integers(1, 4)), int(rng.integers(1, 9))
+    cap = rng.integers(1, 3000, size=Hkv)
+    gaps = rng.integers(0, 200, size=Hkv + 1)
+    order = rng.permutation(Hkv)
+    start = np.zeros(Hkv, dtype=np.int64)
+    pos = int(gaps[0])
+    for j, h in enumerate(order):
+        start[h] = pos
+        pos += int(cap[h]) + int(gaps[j + 1])
+    sumc = pos
+    hs = np.broadcast_to(start, (B, Hkv)).copy()
+    hv = rng.integers(0, cap + 1, size=(B, Hkv)).astype(np.int64)
+    hv[rng.integers(B), rng.integers(Hkv)] = 0
+    kc = torch.from_numpy(rng.standard_normal((B, sumc, D)).astype(np.float32)).to(dev, dtype)
+    vc = torch.from_numpy(rng.standard_normal((B, sumc, D)).astype(np.float32)).to(dev, dtype)
+    q = torch.from_numpy(rng.standard_normal((B, Hkv * G, 1, D)).astype(np.float32)).to(dev, dtype)
+    out = mixture_of_sparse_attention(q, kc, vc, D ** -0.5, head_start_index=torch.from_numpy(hs).to(dev),
+                                      head_valid_length=torch.from_numpy(hv).to(dev))
+    ref = decode_segments(q[:, :, 0].float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(),
+                          hs, hv, D ** -0.5, group=G)
+    _close(out[:, 0].float().cpu().numpy(), ref, ("random layout", seed, G, D))
+
+
 def test_grouped_query_70b_shape(dev):
     """The 70B shape of the largest config: 64 query heads on 8 rings, head_dim 128, B = 4."""
     from moa_amd import mixture_of_sparse_attention
