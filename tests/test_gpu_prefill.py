@@ -137,14 +137,15 @@ def test_wide_windows_reduce_to_causal(dev):
     _close(out, ref, "causal")
 
 
-def test_gqa(dev):
-    """8 query heads on 2 kv heads: equals MHA with each kv head repeated 4 times."""
-    q, k, v = _qkv(2, 8, 448, 128, torch.float16, dev, seed=5, hkv=2)
+@pytest.mark.parametrize("G", [4, 3])
+def test_gqa(dev, G):
+    """G query heads per kv head (2 kv heads): equals MHA with each kv head repeated G times."""
+    q, k, v = _qkv(2, 2 * G, 448, 128, torch.float16, dev, seed=5, hkv=2)
     ns, nl = [1, 2], [2, 3]
     out = _run(q, k, v, 0.09, ns, nl, dev)
-    kr, vr = k.repeat_interleave(4, dim=1), v.repeat_interleave(4, dim=1)
-    ref = prefill_masked_dense(q, kr, vr, 0.09, [1] * 4 + [2] * 4, [2] * 4 + [3] * 4)
-    _close(out, ref, "gqa")
+    kr, vr = k.repeat_interleave(G, dim=1), v.repeat_interleave(G, dim=1)
+    ref = prefill_masked_dense(q, kr, vr, 0.09, [1] * G + [2] * G, [2] * G + [3] * G)
+    _close(out, ref, ("gqa", G))
 
 
 def test_many_heads_with_equal_and_extreme_spans(dev):
