@@ -692,13 +692,19 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
 #ifndef MOA_DEC_BLOCKS
 #define MOA_DEC_BLOCKS 16
 #endif
+#ifndef MOA_DEC_SMALL_BELOW
+#define MOA_DEC_SMALL_BELOW 2   // work-groups per CU below which the chunks are half as long
+#endif
 #ifndef MOA_DEC_PIPE_FROM
 #define MOA_DEC_PIPE_FROM 3   // work-groups per CU from which the waves pipeline their own loads
 #endif
 constexpr int kChunk = MOA_DEC_CHUNK;
 
-// partial slots per batch row: at most this many chunks exist when the rings do not overlap
-static inline int64_t decode_cap(int64_t sumC, int H) { return (sumC + kChunk - 1) / kChunk + H; }
+constexpr int kSmallChunk = kChunk / 2;   // chunk length of the one-query-head kernel when the grid is small
+
+// partial slots per batch row: at most this many chunks exist when the rings do not overlap (sized
+// for the shortest chunk any of the kernels uses)
+static inline int64_t decode_cap(int64_t sumC, int H) { return (sumC + kSmallChunk - 1) / kSmallChunk + H; }
 // every chunk keeps one partial per query head of its ring
 static inline size_t decode_slots(int B, int Hq, int Hkv, int64_t sumC) {
   return (size_t)B * (size_t)decode_cap(sumC, Hkv) * (size_t)((Hq + Hkv - 1) / Hkv);
@@ -709,12 +715,27 @@ static int launch_decode(const void* q, const void* kc, const void* vc, void* o,
                          float* part_ml, const int64_t* head_start, const int64_t* head_valid, int B,
                          int H, int64_t sumC, float sm_scale, hipStream_t st) {
   const int cap = (int)decode_cap(sumC, H);
+  const int64_t chunks = (sumC + kChunk - 1) / kChunk + H;   // per batch row, at the normal chunk length
   // 16 work-groups per CU over the whole grid (measured: 8 leaves a visible tail, 32 is no better),
   // never more per batch row than chunks exist
   int bx = (int)((256 * MOA_DEC_BLOCKS + B - 1) / B);
   if (bx > cap) bx = cap;
   if (bx < 1) bx = 1;
-  const bool pipe = (int64_t)B * cap >= (int64_t)256 * MOA_DEC_PIPE_FROM;
+  const bool pipe = (int64_t)B * chunks >= (int64_t)256 * MOA_DEC_PIPE_FROM;
+  // fewer than two work-groups per CU: half-length chunks give every CU something to do
+  const bool small = (int64_t)B * chunks < (int64_t)256 * MOA_DEC_SMALL_BELOW;
+  constexpr int GROUPS = kDecThreads / D;
+  const int mx = (H * G + GROUPS - 1) / GROUPS;
+  if (small) {
+    hipLaunchKernelGGL((decode_split_kernel<T, D, kSmallChunk, G, false>), dim3(bx, B), dim3(kDecThreads), 0, st,
+                       (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, (uint16_t*)o,
+                       part_acc, part_ml, head_start, head_valid, H, sumC, sm_scale * kLog2e, cap);
+    int rc = check_launch("moa_decode_fwd(split)");
+    if (rc) return rc;
+    hipLaunchKernelGGL((decode_merge_kernel<T, D, kSmallChunk>), dim3(mx, B), dim3(kDecThreads), 0, st,
+                       (uint16_t*)o, part_acc, part_ml, head_valid, H, G, cap);
+    return check_launch("moa_decode_fwd(merge)");
+  }
   if (pipe)
     hipLaunchKernelGGL((decode_split_kernel<T, D, kChunk, G, true>), dim3(bx, B), dim3(kDecThreads), 0, st,
                        (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, (uint16_t*)o,
@@ -725,8 +746,6 @@ static int launch_decode(const void* q, const void* kc, const void* vc, void* o,
                        part_acc, part_ml, head_start, head_valid, H, sumC, sm_scale * kLog2e, cap);
   int rc = check_launch("moa_decode_fwd(split)");
   if (rc) return rc;
-  constexpr int GROUPS = kDecThreads / D;
-  int mx = (H * G + GROUPS - 1) / GROUPS;
   hipLaunchKernelGGL((decode_merge_kernel<T, D, kChunk>), dim3(mx, B), dim3(kDecThreads), 0, st,
                      (uint16_t*)o, part_acc, part_ml, head_valid, H, G, cap);
   return check_launch("moa_decode_fwd(merge)");

@@ -89,13 +89,15 @@ def test_partial_fill_and_empty_heads(dev, dtype):
     assert not out[0, 0].any() and not out[1, 3].any()
 
 
+@pytest.mark.parametrize("B", [64, 40])
 @pytest.mark.parametrize("D", [128, 64])
-def test_partial_fill_with_a_large_grid(dev, D):
-    """Enough work-groups (batch 64) that the kernel takes its load-pipelined loop: ragged valid
-    lengths, an empty head, lengths around the half-batch of rows that loop works in."""
-    rng = np.random.default_rng(77 + D)
+def test_partial_fill_with_a_large_grid(dev, D, B):
+    """Grids beyond the small-grid variant (half-length chunks): batch 64 takes the load-pipelined
+    loop, batch 40 the plain loop with full-length chunks.  Ragged valid lengths, an empty head,
+    lengths around the half-batch of rows the pipelined loop works in."""
+    rng = np.random.default_rng(77 + D + B)
     sizes = [64, 576, 1344, 192, 2112, 128]
-    q, kc, vc, hs, hv = _case(rng, 64, sizes, D, torch.float16, dev, fill="partial")
+    q, kc, vc, hs, hv = _case(rng, B, sizes, D, torch.float16, dev, fill="partial")
     hv[0, :] = [1, 15, 16, 17, 33, 0]
     hv[1, :] = [31, 32, 63, 64, 65, 127]
     out, ref = _run(q, kc, vc, hs, hv, D ** -0.5, dev)
