@@ -37,8 +37,13 @@ def test_header_symbols_exported(lib):
 
 def test_host_only_entry_points(lib):
     assert lib.moa_abi_version() == 1
-    # decode workspace: (ceil(sumC/512) + H) partial slots per batch row, D+2 floats each
-    assert lib.moa_decode_workspace_bytes(2, 4, 4, 128, 1024) == 2 * (2 + 4) * 130 * 4 // 256 * 256 + (256 if (2 * 6 * 130 * 4) % 256 else 0)
+    # decode workspace: (ceil(sumC/256) + Hkv) * (Hq/Hkv) partial slots per batch row, D+2 floats each,
+    # rounded up to 256 bytes
+    def expect(B, Hq, Hkv, D, sumC):
+        raw = B * (-(-sumC // 256) + Hkv) * (Hq // Hkv) * (D + 2) * 4
+        return -(-raw // 256) * 256
+    assert lib.moa_decode_workspace_bytes(2, 4, 4, 128, 1024) == expect(2, 4, 4, 128, 1024)
+    assert lib.moa_decode_workspace_bytes(3, 16, 2, 64, 5000) == expect(3, 16, 2, 64, 5000)
     assert lib.moa_decode_workspace_bytes(0, 4, 4, 128, 1024) == 0
     assert lib.moa_cache_prefill_workspace_bytes(3, 100) >= 3 * 201 * 4
 
