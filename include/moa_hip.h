@@ -104,6 +104,25 @@ int moa_decode_fwd(const void* q, const void* kc, const void* vc, void* o,
                    float sm_scale, int dtype, void* stream);
 
 /*
+ * moa_decode_fwd without a workspace argument, for callers that cannot allocate
+ * device memory: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  It has no counterpart in the reference.  Same
+ * arguments, kernels and results as moa_decode_fwd; the split-K partials go
+ * into a scratch array of MOA_DECODE_NOALLOC_MAX_BYTES that is part of the
+ * library's device image (every GPU the library runs on holds it until the
+ * process ends).  Sizes for which moa_decode_workspace_bytes(...) exceeds that
+ * are rejected with MOA_ERR_WORKSPACE.  The call allocates and frees nothing.
+ * All calls on one GPU share that GPU's array: calls that may overlap on one
+ * GPU (different streams, different threads) race on it and must be
+ * serialised by the caller.
+ */
+#define MOA_DECODE_NOALLOC_MAX_BYTES (32u << 20)
+int moa_decode_fwd_noalloc(const void* q, const void* kc, const void* vc, void* o,
+                           const int64_t* head_start, const int64_t* head_valid_len,
+                           int B, int Hq, int Hkv, int D, int64_t sumC,
+                           float sm_scale, int dtype, void* stream);
+
+/*
  * One decode-step append into every head's ring, with the index bookkeeping,
  * in one launch.
  * Replaces: the decode branch of StaticCircularCache.update

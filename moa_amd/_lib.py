@@ -23,6 +23,8 @@ MOA_DTYPE_F16 = 0
 MOA_DTYPE_BF16 = 1
 MOA_DTYPE_F32 = 2
 
+MOA_DECODE_NOALLOC_MAX_BYTES = 32 << 20
+
 ABI_VERSION = 1
 
 # name -> (restype, argtypes); must list every symbol include/moa_hip.h declares
@@ -36,6 +38,8 @@ SIGNATURES = {
     "moa_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int64]),
     "moa_decode_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p,
                                c_void_p, c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_void_p]),
+    "moa_decode_fwd_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                       c_int, c_int, c_int64, c_float, c_int, c_void_p]),
     "moa_cache_append": (c_int, [c_void_p, c_void_p, _I64P, _I64P, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
                                  c_int, c_int64, c_int, c_void_p]),

@@ -31,6 +31,8 @@
 
 #include <hip/hip_fp16.h>
 
+#include <mutex>
+
 namespace moa {
 
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
@@ -777,37 +779,13 @@ static int launch_decode_gqa(const void* q, const void* kc, const void* vc, void
   return check_launch("moa_decode_fwd(merge)");
 }
 
-}  // namespace moa
-
-using namespace moa;
-
-extern "C" size_t moa_decode_workspace_bytes(int B, int Hq, int Hkv, int D, int64_t sumC) {
-  if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || sumC <= 0) return 0;
-  const size_t slots = decode_slots(B, Hq, Hkv, sumC);
-  return ((slots * ((size_t)D + 2) * sizeof(float)) + 255) & ~(size_t)255;
-}
-
-extern "C" int moa_decode_fwd(const void* q, const void* kc, const void* vc, void* o, void* workspace,
-                              size_t workspace_bytes, const int64_t* head_start,
-                              const int64_t* head_valid_len, int B, int Hq, int Hkv, int D, int64_t sumC,
-                              float sm_scale, int dtype, void* stream) {
-  if (!q || !kc || !vc || !o || !head_start || !head_valid_len)
-    return fail(MOA_ERR_ARG, "moa_decode_fwd: null pointer");
-  if (B <= 0 || Hq <= 0 || Hkv <= 0 || sumC <= 0) return fail(MOA_ERR_ARG, "moa_decode_fwd: B, H, sumC must be positive");
-  if (B > 65535) return fail(MOA_ERR_UNSUPPORTED, "moa_decode_fwd: B <= 65535");
-  if (Hq % Hkv != 0) return fail(MOA_ERR_ARG, "moa_decode_fwd: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
+// Launches the decode kernels with their partials in `workspace` (at least
+// moa_decode_workspace_bytes(...) bytes; arguments and size are checked by the entry points).
+static int decode_dispatch(const void* q, const void* kc, const void* vc, void* o,
+                           void* workspace, const int64_t* head_start, const int64_t* head_valid_len,
+                           int B, int Hq, int Hkv, int D, int64_t sumC, float sm_scale, int dtype,
+                           void* stream) {
   const int G = Hq / Hkv;
-  if (G > kGqaMaxG)
-    return fail(MOA_ERR_UNSUPPORTED, "moa_decode_fwd: %d query heads per kv head (at most %d)", G, kGqaMaxG);
-  if (Hkv > kMaxHeads) return fail(MOA_ERR_UNSUPPORTED, "moa_decode_fwd: at most %d kv heads", kMaxHeads);
-  if (D != 64 && D != 128) return fail(MOA_ERR_UNSUPPORTED, "moa_decode_fwd: head_dim %d (64 or 128)", D);
-  if (dtype != MOA_DTYPE_F16 && dtype != MOA_DTYPE_BF16)
-    return fail(MOA_ERR_UNSUPPORTED, "moa_decode_fwd: dtype %d (f16 or bf16)", dtype);
-  if (!aligned16(q) || !aligned16(kc) || !aligned16(vc) || !aligned16(o))
-    return fail(MOA_ERR_ARG, "moa_decode_fwd: pointers must be 16-byte aligned");
-  const size_t need = moa_decode_workspace_bytes(B, Hq, Hkv, D, sumC);
-  if (!workspace || workspace_bytes < need)
-    return fail(MOA_ERR_WORKSPACE, "moa_decode_fwd: workspace %zu < %zu bytes", workspace_bytes, need);
   const size_t slots = decode_slots(B, Hq, Hkv, sumC);
   float* part_acc = reinterpret_cast<float*>(workspace);
   float* part_ml = part_acc + slots * (size_t)D;
@@ -823,4 +801,88 @@ extern "C" int moa_decode_fwd(const void* q, const void* kc, const void* vc, voi
   return G == 1 ? launch_decode<BF16, 64, 1>(MOA_DEC_ARGS, MOA_DEC_TAIL) : launch_decode_gqa<BF16, 64>(MOA_DEC_ARGS, G, MOA_DEC_TAIL);
 #undef MOA_DEC_TAIL
 #undef MOA_DEC_ARGS
+}
+
+static int decode_check_args(const char* who, const void* q, const void* kc, const void* vc, const void* o,
+                             const int64_t* head_start, const int64_t* head_valid_len, int B, int Hq,
+                             int Hkv, int D, int64_t sumC, int dtype) {
+  if (!q || !kc || !vc || !o || !head_start || !head_valid_len) return fail(MOA_ERR_ARG, "%s: null pointer", who);
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || sumC <= 0) return fail(MOA_ERR_ARG, "%s: B, H, sumC must be positive", who);
+  if (B > 65535) return fail(MOA_ERR_UNSUPPORTED, "%s: B <= 65535", who);
+  if (Hq % Hkv != 0) return fail(MOA_ERR_ARG, "%s: Hq=%d is not a multiple of Hkv=%d", who, Hq, Hkv);
+  const int G = Hq / Hkv;
+  if (G > kGqaMaxG) return fail(MOA_ERR_UNSUPPORTED, "%s: %d query heads per kv head (at most %d)", who, G, kGqaMaxG);
+  if (Hkv > kMaxHeads) return fail(MOA_ERR_UNSUPPORTED, "%s: at most %d kv heads", who, kMaxHeads);
+  if (D != 64 && D != 128) return fail(MOA_ERR_UNSUPPORTED, "%s: head_dim %d (64 or 128)", who, D);
+  if (dtype != MOA_DTYPE_F16 && dtype != MOA_DTYPE_BF16) return fail(MOA_ERR_UNSUPPORTED, "%s: dtype %d (f16 or bf16)", who, dtype);
+  if (!aligned16(q) || !aligned16(kc) || !aligned16(vc) || !aligned16(o))
+    return fail(MOA_ERR_ARG, "%s: pointers must be 16-byte aligned", who);
+  return MOA_OK;
+}
+
+// ---- scratch of the entry point that allocates nothing -------------------------------------------
+// The split-K partials of moa_decode_fwd_noalloc live in this file-scope array instead of a caller's
+// workspace.  Every GPU the library runs on holds its own copy at its own address until the process
+// ends.  In host code the array's name is only a handle for hipGetSymbolAddress: the kernels get the
+// device address looked up below, once per device.
+static __device__ __align__(256) unsigned char scratch[MOA_DECODE_NOALLOC_MAX_BYTES];
+
+static int noalloc_scratch(void** out) {
+  static void* ptr_of_device[kMaxDevices] = {};
+  static std::mutex mu;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(MOA_ERR_LAUNCH, "moa_decode_fwd_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(MOA_ERR_UNSUPPORTED, "moa_decode_fwd_noalloc: device %d (at most %d devices)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptr_of_device[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));   // the copy of the array on the current device
+    if (e != hipSuccess || !p)
+      return fail(MOA_ERR_LAUNCH, "moa_decode_fwd_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    ptr_of_device[dev] = p;
+  }
+  *out = ptr_of_device[dev];
+  return MOA_OK;
+}
+
+}  // namespace moa
+
+using namespace moa;
+
+extern "C" size_t moa_decode_workspace_bytes(int B, int Hq, int Hkv, int D, int64_t sumC) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || sumC <= 0) return 0;
+  const size_t slots = decode_slots(B, Hq, Hkv, sumC);
+  return ((slots * ((size_t)D + 2) * sizeof(float)) + 255) & ~(size_t)255;
+}
+
+extern "C" int moa_decode_fwd(const void* q, const void* kc, const void* vc, void* o, void* workspace,
+                              size_t workspace_bytes, const int64_t* head_start,
+                              const int64_t* head_valid_len, int B, int Hq, int Hkv, int D, int64_t sumC,
+                              float sm_scale, int dtype, void* stream) {
+  if (int rc = decode_check_args("moa_decode_fwd", q, kc, vc, o, head_start, head_valid_len, B, Hq, Hkv, D, sumC, dtype))
+    return rc;
+  const size_t need = moa_decode_workspace_bytes(B, Hq, Hkv, D, sumC);
+  if (!workspace || workspace_bytes < need)
+    return fail(MOA_ERR_WORKSPACE, "moa_decode_fwd: workspace %zu < %zu bytes", workspace_bytes, need);
+  return decode_dispatch(q, kc, vc, o, workspace, head_start, head_valid_len, B, Hq, Hkv, D,
+                         sumC, sm_scale, dtype, stream);
+}
+
+extern "C" int moa_decode_fwd_noalloc(const void* q, const void* kc, const void* vc, void* o,
+                                      const int64_t* head_start, const int64_t* head_valid_len, int B,
+                                      int Hq, int Hkv, int D, int64_t sumC, float sm_scale, int dtype,
+                                      void* stream) {
+  if (int rc = decode_check_args("moa_decode_fwd_noalloc", q, kc, vc, o, head_start, head_valid_len, B, Hq, Hkv, D, sumC, dtype))
+    return rc;
+  const size_t need = moa_decode_workspace_bytes(B, Hq, Hkv, D, sumC);
+  if (need > (size_t)MOA_DECODE_NOALLOC_MAX_BYTES)
+    return fail(MOA_ERR_WORKSPACE,
+                "moa_decode_fwd_noalloc: these sizes need %zu bytes of partials, the built-in scratch holds %zu; "
+                "use moa_decode_fwd with a workspace",
+                need, (size_t)MOA_DECODE_NOALLOC_MAX_BYTES);
+  void* ws = nullptr;
+  if (int rc = noalloc_scratch(&ws)) return rc;
+  return decode_dispatch(q, kc, vc, o, ws, head_start, head_valid_len, B, Hq, Hkv, D,
+                         sumC, sm_scale, dtype, stream);
 }
