@@ -463,8 +463,11 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     uint16_t* __restrict__ o, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const int64_t* __restrict__ head_start, const int64_t* __restrict__ head_valid, int H,
-    int G /* query heads per ring, <= kGqaMaxG */, int64_t sumC, float scale_log2, int cap) {
+    int G /* query heads per ring, <= kGqaMaxG */, int64_t sumC, float scale_log2_signed, int cap) {
   typedef typename MfmaElem<T>::type M;
+  // the row maximum is taken over unscaled scores: a negative softmax scale goes into Q (sign flip, exact)
+  const float scale_log2 = __builtin_fabsf(scale_log2_signed);
+  const uint32_t q_sign = scale_log2_signed < 0.f ? 0x80008000u : 0u;
   constexpr int KS = D / 16;                    // MFMA k-steps of Q.K^T
   constexpr int DT = D / 32;                    // 32-wide d tiles of the output
   constexpr int CPR = D / 8;                    // 16-byte chunks per cache row
@@ -542,6 +545,7 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
     for (int s = 0; s < KS; ++s) {
       u32x4 z = {0, 0, 0, 0};
       qf[s] = (mcol < G) ? *reinterpret_cast<const u32x4*>(q + (bh * G + mcol) * D + 16 * s + 8 * g) : z;
+      qf[s] ^= u32x4{q_sign, q_sign, q_sign, q_sign};
     }
     f32x16 oacc[DT];
 #pragma unroll
@@ -608,7 +612,8 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
       mx = max_with_other_half(mx);
       const float m_cand = mx * scale_log2;   // finite: key 0 of the tile is valid
       if (__any(m_cand > m_run + kRescaleStep)) {
-        const float m_new = fmaxf(m_run, m_cand);
+        // an integer reference exponent: the rounding of the weights below is then independent of it
+        const float m_new = __builtin_ceilf(fmaxf(m_run, m_cand));
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         l_run *= alpha;
 #pragma unroll
@@ -769,7 +774,7 @@ static int launch_decode_gqa(const void* q, const void* kc, const void* vc, void
     return rc;
   hipLaunchKernelGGL((decode_gqa_kernel<T, D>), dim3(bx, B), dim3(kGqaThreads), lds, st,
                      (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, (uint16_t*)o,
-                     part_acc, part_ml, head_start, head_valid, H, G, sumC, sm_scale * kLog2e, cap);
+                     part_acc, part_ml, head_start, head_valid, H, G, sumC, mfma_softmax_scale(sm_scale), cap);
   int rc = check_launch("moa_decode_fwd(grouped split)");
   if (rc) return rc;
   constexpr int GROUPS = kDecThreads / D;

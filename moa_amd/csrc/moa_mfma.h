@@ -84,6 +84,14 @@ __device__ __forceinline__ void phase_barrier() {
   asm volatile("" ::: "memory");
 }
 
+// sm_scale * log2(e) as the MFMA kernels take it.  They mask a score by setting it to -inf before
+// the multiply-add with the scale, and -inf * 0 is NaN: a scale of exactly zero (uniform weights) is
+// replaced by one so small that every finite score still maps to 2^0 = 1 exactly.
+inline float mfma_softmax_scale(float sm_scale) {
+  const float s = sm_scale * 1.4426950408889634f;
+  return s == 0.f ? 1e-30f : s;
+}
+
 template <int P>
 struct IC {
   static constexpr int value = P;

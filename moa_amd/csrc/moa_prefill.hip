@@ -52,7 +52,6 @@ constexpr int kWRows = 32;    // query rows per wave
 constexpr int kKV = 64;       // keys per tile (the sparsity block)
 constexpr int kStages = 4;    // LDS stages per tensor
 constexpr int kMaxSortedHeads = 512;   // kv heads the span-sorted schedule handles (else: given order)
-constexpr float kLog2eF = 1.4426950408889634f;
 
 struct Strides4 {
   int64_t b, h, n;
@@ -63,7 +62,7 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
     uint16_t* __restrict__ o, Strides4 qs, Strides4 ks, Strides4 vs, Strides4 os, int BH, int Hq,
     int group, int N, int n_qtiles, const int64_t* __restrict__ sink_blocks,
-    const int64_t* __restrict__ local_blocks, float scale_log2) {
+    const int64_t* __restrict__ local_blocks, float scale_log2_signed) {
   constexpr int KS = D / 16;          // MFMA k-steps of the QK^T product
   constexpr int DT = D / 32;          // 32-wide d tiles of the output
   constexpr int CPR = D / 8;          // 16-byte chunks per K/V row
@@ -72,6 +71,10 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
   constexpr int ROW_B = D * 2;
   constexpr int RSH = 16 / CPR;       // rows per 256 bytes of LDS (1 at D=128, 2 at D=64)
   constexpr float kRescaleStep = 8.f; // rescale O only when a row max grew by more than 2^8
+  // The row maximum is taken over the unscaled scores, which needs a scale >= 0: a negative softmax
+  // scale is moved into Q (sign bits of the packed 16-bit elements flipped, exact) and its magnitude kept.
+  const float scale_log2 = __builtin_fabsf(scale_log2_signed);
+  const uint32_t q_sign = scale_log2_signed < 0.f ? 0x80008000u : 0u;
   static_assert(4 * DT == 2 * KS, "P.V and Q.K^T have the same number of MFMAs per tile");
 
   // LDS: kStages K stages, then kStages V stages; tile t lives in stage t % kStages.  Rows are
@@ -243,6 +246,7 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
     for (int s = 0; s < KS; ++s) {
       u32x4 z = {0, 0, 0, 0};
       qf[s] = ok ? *reinterpret_cast<const u32x4*>(qrow + 16 * s) : z;
+      qf[s] ^= u32x4{q_sign, q_sign, q_sign, q_sign};
     }
   }
 
@@ -255,7 +259,7 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
   uint32_t pf[16];           // P^T of the current tile, packed pairs, B-operand order
 #pragma unroll
   for (int i = 0; i < 16; ++i) pf[i] = 0;
-  float m_run = -INFINITY;   // reference max of scale_log2 * s used by exp2 (lags the true max by <= kRescaleStep)
+  float m_run = -INFINITY;   // reference exponent of exp2: an integer >= the max of scale_log2 * s when set, then lagging it by <= kRescaleStep
   float l_run = 0.f;         // this lane's share of the running sum (the lane+32 twin holds the rest)
 
   // ---- operand read addresses: LDS byte address of stage 0, row 0 of this lane; stage, half and
@@ -357,7 +361,10 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
     mx = max_with_other_half(mx);
     const float m_cand = mx * scale_log2;   // finite: a live tile has a visible key in every row
     if (__any(m_cand > m_run + kRescaleStep)) {
-      const float m_new = fmaxf(m_run, m_cand);
+      // The reference exponent stays an INTEGER: a weight is then 2^frac * 2^int, and its rounding to the
+      // storage type below does not depend on the power of two, so the rounded weights (relative to the
+      // row's sum) do not depend on the tile order or on how far m_run lags behind the true maximum.
+      const float m_new = __builtin_ceilf(fmaxf(m_run, m_cand));
       const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
       l_run *= alpha;
 #pragma unroll
@@ -490,7 +497,7 @@ static int launch_prefill(const void* q, const void* k, const void* v, void* o, 
     return rc;
   hipLaunchKernelGGL((prefill_kernel<T, D>), dim3((unsigned)groups), dim3(kPfThreads), lds, st,
                      (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (uint16_t*)o, sq, sk, sv,
-                     so, BH, Hq, Hq / Hkv, N, n_qtiles, sink_blocks, local_blocks, sm_scale * kLog2eF);
+                     so, BH, Hq, Hq / Hkv, N, n_qtiles, sink_blocks, local_blocks, mfma_softmax_scale(sm_scale));
   return check_launch("moa_prefill_fwd");
 }
 

@@ -22,6 +22,10 @@ reference checkout).  What pins each function (see tests/test_oracle_*.py):
   prefill_blockwise                 follows the kernel's block loop and its
       base-2 incremental softmax; checked against prefill_masked_dense and a
       brute-force triple loop.
+  prefill_p_rounded                 the same attention with the softmax weights rounded to the
+      storage type in front of P.V (where the reference's kernel rounds them); equals
+      prefill_masked_dense without rounding, a pure-Python loop that rounds through torch's
+      casts on a tiny input, and itself under integer shifts of the reference exponent.
   decode_segments                   closed form; checked against
       decode_grouped_sdpa (the reference's grouped-SDPA decode), ring-order
       invariance and prefill/decode consistency.
@@ -233,6 +237,70 @@ def prefill_bruteforce(q: np.ndarray, k: np.ndarray, v: np.ndarray, sm_scale: fl
     return out
 
 
+def round_to_storage(x: np.ndarray, p_dtype: Optional[str]) -> np.ndarray:
+    """fp32 values rounded to nearest-even into ``"bf16"`` (8 significant bits) or ``"f16"`` (11 bits,
+    subnormals below 2^-14), returned as fp32; ``None`` returns ``x`` unchanged.  bf16 is done on the
+    bit pattern (add 0x7fff + lsb, truncate), independent of any library's cast."""
+    x = np.asarray(x, dtype=np.float32)
+    if p_dtype is None:
+        return x
+    if p_dtype == "f16":
+        return x.astype(np.float16).astype(np.float32)
+    assert p_dtype == "bf16", p_dtype
+    u = x.view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32).reshape(x.shape)
+
+
+def prefill_p_rounded(q, k, v, sm_scale: float, sink_blocks, local_blocks, p_dtype: Optional[str],
+                      block: int = BLOCK, shift: int = 0, rows_per_step: int = 1024) -> np.ndarray:
+    """Masked attention whose softmax weights enter the P.V product ROUNDED to the storage type,
+    the place where the reference's kernel rounds them (``p.to(tl.float16)`` in front of
+    ``tl.dot(p, v)``, MoA/kernels/block_sparse_attention_prefill.py:608-610), everything else exact:
+
+        t_ij = log2(e) * sm_scale * (q_i . k_j)                       fp64
+        M_i  = ceil(max_j t_ij) + shift                                an integer
+        p_ij = fp32(2^(t_ij - M_i))                                    unnormalised weight
+        o_i  = sum_j round(p_ij) v_j / sum_j p_ij                      the sum of weights is NOT rounded (:590)
+
+    Because M_i is an integer, round() is applied to 2^frac * 2^int and the rounding of a binary
+    floating-point format does not depend on the power of two: the result is the same for every
+    integer ``shift`` (while nothing over- or underflows) and therefore does not depend on the order
+    in which an online-softmax kernel meets the keys, as long as that kernel keeps its running
+    reference exponent integral.  The reference's own kernel rounds the weight scaled by a
+    non-integral running normaliser instead (:593-609); the two differ by independent rounding
+    errors of the same size (relative 2^-8 per weight for bf16, 2^-11 for f16).
+
+    q, k, v: torch tensors or arrays [B, H, N, D]; returns fp64 [B, H, N, D].  ``p_dtype=None``
+    rounds nothing and equals prefill_masked_dense.  Rows with no visible key return 0.
+    """
+    def arr(t):
+        if hasattr(t, "detach"):
+            t = t.detach().float().cpu().numpy()
+        return np.asarray(t, dtype=np.float64)
+
+    qa, ka, va = arr(q), arr(k), arr(v)
+    B, H, N, D = qa.shape
+    out = np.zeros((B, H, N, D), dtype=np.float64)
+    c = sm_scale * 1.4426950408889634
+    for h in range(H):
+        mask = moa_token_mask(N, int(sink_blocks[h]), int(local_blocks[h]), block)
+        for b in range(B):
+            for r0 in range(0, N, rows_per_step):
+                r1 = min(N, r0 + rows_per_step)
+                m = mask[r0:r1, :r1]                       # causal: no key beyond the last row of the step
+                t = (qa[b, h, r0:r1] @ ka[b, h, :r1].T) * c
+                t = np.where(m, t, -np.inf)
+                alive = m.any(axis=1)
+                M = np.where(alive, np.ceil(np.max(t, axis=1, initial=-np.inf, where=m)), 0.0) + shift
+                p = np.exp2(t - M[:, None]).astype(np.float32)
+                l = p.astype(np.float64).sum(axis=1)
+                pr = round_to_storage(p, p_dtype).astype(np.float64)
+                o = pr @ va[b, h, :r1]
+                out[b, h, r0:r1] = np.where(alive[:, None], o / np.where(alive, l, 1.0)[:, None], 0.0)
+    return out
+
+
 # --------------------------------------------------------------------------
 # Decode arithmetic
 # --------------------------------------------------------------------------
@@ -240,13 +308,19 @@ def prefill_bruteforce(q: np.ndarray, k: np.ndarray, v: np.ndarray, sm_scale: fl
 
 def decode_segments(q: np.ndarray, kc: np.ndarray, vc: np.ndarray,
                     head_start: np.ndarray, head_valid: np.ndarray,
-                    sm_scale: float, group: int = 1) -> np.ndarray:
+                    sm_scale: float, group: int = 1, p_dtype: Optional[str] = None,
+                    abs_v: bool = False) -> np.ndarray:
     """Per (b, h): softmax(sm_scale * q . K_seg^T) V_seg over rows
     [start[b,hk], start[b,hk] + valid[b,hk]) of the packed cache; no mask.
 
     q [B, Hq, D]; kc, vc [B, sumC, D]; head_start/head_valid [B, Hkv] int64;
     query head h reads kv head h // group.  fp64.  Returns [B, Hq, D].
     A head with valid == 0 returns 0.
+
+    ``p_dtype`` ("bf16" / "f16"): the weights enter the product with V rounded to that type, with
+    the integral reference exponent of prefill_p_rounded (same formula, same reasons); the
+    grouped-query kernel works like that.  ``abs_v``: attend to |V| (the scale of a weight-rounding
+    error bound).
 
     Semantics of the external decode op as used at
     MoA/kernels/mixture_of_attention.py:465-473 (argument docs :389-392), and of
@@ -263,10 +337,17 @@ def decode_segments(q: np.ndarray, kc: np.ndarray, vc: np.ndarray,
                 continue
             ks = kc[b, s0:s0 + n].astype(np.float64)
             vs = vc[b, s0:s0 + n].astype(np.float64)
+            if abs_v:
+                vs = np.abs(vs)
             s = ks @ q[b, h].astype(np.float64) * sm_scale
-            s -= s.max()
-            p = np.exp(s)
-            out[b, h] = (p / p.sum()) @ vs
+            if p_dtype is None:
+                s -= s.max()
+                p = np.exp(s)
+                out[b, h] = (p / p.sum()) @ vs
+            else:
+                t = s * 1.4426950408889634
+                p = np.exp2(t - np.ceil(t.max())).astype(np.float32)
+                out[b, h] = (round_to_storage(p, p_dtype).astype(np.float64) @ vs) / p.astype(np.float64).sum()
     return out
 
 

@@ -9,7 +9,7 @@ import torch.nn.functional as F
 from oracle.moa_oracle import (count_live_pairs, decode_grouped_sdpa, decode_segments,
                                live_kv_blocks, moa_token_mask, moa_token_mask_from_blocks,
                                prefill_blockwise, prefill_bruteforce, prefill_masked_dense,
-                               head_start_valid_to_head_index)
+                               prefill_p_rounded, round_to_storage, head_start_valid_to_head_index)
 
 
 def test_mask_two_formulations_agree_exhaustively():
@@ -106,6 +106,60 @@ def test_prefill_invariants():
     torch.testing.assert_close(o2, o, rtol=1e-4, atol=1e-5)
 
 
+def test_round_to_storage_against_torch_casts():
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(20000) * 10.0 ** rng.integers(-8, 3, 20000),
+                        [0.0, 1.0, 1.00390625, 1.01171875, 256.0, 2.0 ** -20, 3.0 * 2.0 ** -26]]).astype(np.float32)
+    for name, dt in (("bf16", torch.bfloat16), ("f16", torch.float16)):
+        mine = round_to_storage(x, name)
+        theirs = torch.from_numpy(x).to(dt).float().numpy()
+        assert np.array_equal(mine, theirs), name
+    # ties go to the even neighbour: 1 + 2^-8 -> 1, 1 + 3 * 2^-8 -> 1 + 2^-6 (bf16 spacing at 1 is 2^-7)
+    assert round_to_storage(np.float32([1.00390625, 1.01171875]), "bf16").tolist() == [1.0, 1.015625]
+    assert round_to_storage(x, None) is not None and np.array_equal(round_to_storage(x, None), x)
+
+
+def test_p_rounded_prefill_is_pinned():
+    """(1) without rounding it is the masked dense attention; (2) with rounding it equals a
+    pure-Python evaluation of its defining formula that rounds through torch's scalar casts;
+    (3) integer shifts of the reference exponent change nothing (bit for bit in the weights,
+    to fp64 rounding in the output); (4) the rounding moves the result by no more than
+    u * (attention of |V| + ...) with u = 2^-8 (bf16) / 2^-11 (f16)."""
+    B, H, N, D = 1, 3, 192, 16
+    q, k, v = (_rand((B, H, N, D), s) for s in (20, 21, 22))
+    ns, nl = [1, 0, 2], [1, 2, 1]
+    sm = 0.3
+    exact = prefill_masked_dense(q, k, v, sm, ns, nl).numpy()
+    none = prefill_p_rounded(q, k, v, sm, ns, nl, None)
+    assert np.abs(none - exact).max() < 2e-6
+    absv = prefill_p_rounded(q, k, v.abs(), sm, ns, nl, None)
+    for name, dt, u in (("bf16", torch.bfloat16, 2.0 ** -8), ("f16", torch.float16, 2.0 ** -11)):
+        got = prefill_p_rounded(q, k, v, sm, ns, nl, name, rows_per_step=80)
+        # (2) brute force, head 0 and 2, a few rows incl. the first of a block
+        c = sm * 1.4426950408889634
+        for h in (0, 2):
+            for i in (0, 1, 63, 64, 65, 130, 191):
+                js = [j for j in range(i + 1) if (j // 64) < ns[h] or (j // 64) >= (i // 64) + 1 - nl[h]]
+                t = [c * float(np.dot(q[0, h, i].double().numpy(), k[0, h, j].double().numpy())) for j in js]
+                M = float(np.ceil(max(t)))
+                p32 = [np.float32(2.0 ** (x - M)) for x in t]
+                den = sum(float(x) for x in p32)
+                o = np.zeros(D)
+                for pj, j in zip(p32, js):
+                    w = float(torch.tensor(float(pj), dtype=torch.float32).to(dt).float())
+                    o += w * v[0, h, j].double().numpy()
+                assert np.abs(o / den - got[0, h, i]).max() < 1e-12, (name, h, i)
+        # (3) shift invariance: exact in bf16 up to the fp32 evaluation of 2^x (1e-8 relative per weight);
+        # f16 rounds weights below 2^-14 on its subnormal grid (spacing 2^-24), which a shift moves:
+        # up to 2^-25 * 2^shift per key, relative to a weight sum of about 1
+        for shift in (-3, 5):
+            shifted = prefill_p_rounded(q, k, v, sm, ns, nl, name, shift=shift)
+            assert np.abs(shifted - got).max() < (1e-8 if name == "bf16" else 1e-4), (name, shift)
+        # (4) the a-priori bound of the weight rounding
+        assert (np.abs(got - none) <= u * absv + 1e-9).all(), name
+        assert np.abs(got - none).max() > 0.05 * u, name     # and the rounding is really there
+
+
 def _packed_case(seed, B=2, sizes=(64, 64, 128, 192, 192), D=16, full=True):
     rng = np.random.default_rng(seed)
     sizes = np.asarray(sizes)
@@ -172,6 +226,25 @@ def test_decode_equals_token_granular_prefill_row():
     sc = np.where(m, sc, -np.inf)
     w = np.exp(sc - sc.max()); w /= w.sum()
     assert np.abs(o - w @ v).max() < 1e-12
+
+
+def test_decode_rounded_weights_match_the_prefill_formulation():
+    """decode_segments(p_dtype=...) is prefill_p_rounded's formula on one query row: the row of a
+    prompt that sees every key (a wide window) gives the same numbers."""
+    rng = np.random.default_rng(12)
+    N, D = 150, 16
+    q, k, v = (rng.standard_normal((1, 1, N, D)).astype(np.float32) for _ in range(3))
+    for name in ("bf16", "f16", None):
+        full = prefill_p_rounded(q, k, v, 0.3, [0], [99], name)[0, 0, N - 1]
+        dec = decode_segments(q[:, :, N - 1], k[0], v[0], np.array([[0]]), np.array([[N]]), 0.3, p_dtype=name)[0, 0]
+        # (without rounding the prefill function still carries its weights in fp32, the decode one in fp64)
+        assert np.abs(full - dec).max() < (1e-12 if name else 1e-7), name
+    # and the weight rounding moves the result by no more than u * attention(|V|)
+    exact = decode_segments(q[:, :, N - 1], k[0], v[0], np.array([[0]]), np.array([[N]]), 0.3)
+    absv = decode_segments(q[:, :, N - 1], k[0], v[0], np.array([[0]]), np.array([[N]]), 0.3, abs_v=True)
+    for name, u in (("bf16", 2.0 ** -8), ("f16", 2.0 ** -11)):
+        dec = decode_segments(q[:, :, N - 1], k[0], v[0], np.array([[0]]), np.array([[N]]), 0.3, p_dtype=name)
+        assert (np.abs(dec - exact) <= u * absv + 1e-9).all() and np.abs(dec - exact).max() > 0
 
 
 def test_decode_gqa_group():

@@ -73,8 +73,11 @@ def _check(q, kc, vc, hs, hv, G, dev, tag):
     o_na, o_ws = _both(q, kc, vc, hs, hv, sm, dev)
     assert torch.isfinite(o_na.float()).all(), tag
     assert torch.equal(o_na, o_ws), (tag, (o_na.float() - o_ws.float()).abs().max().item())
+    # with several query heads per ring the kernel rounds the softmax weights to the input type in front
+    # of P.V; the oracle does it at the same place
+    name = None if G == 1 else ("bf16" if q.dtype == torch.bfloat16 else "f16")
     ref = decode_segments(q.float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(), hs, hv, sm,
-                          group=G)
+                          group=G, p_dtype=name)
     err = np.abs(o_na.float().cpu().numpy() - ref)
     assert (err <= ATOL + RTOL * np.abs(ref)).all(), (tag, float(err.max()))
 
