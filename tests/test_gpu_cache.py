@@ -55,6 +55,12 @@ def test_reference_vectors_on_gpu(dev, golden_dir):
         H = len(case["cache_size"])
         cache = StaticCircularCache([case["cache_size"]], static_size=[case["static_size"]], batch_size=B,
                                     head_dim=D, device=dev, dtype=torch.float32)
+        ctor = case["ctor"]   # what the reference's constructor builds (cache_utils.py:698-769)
+        assert cache.cache_head_start_index[0].tolist() == ctor["head_start"], case["name"]
+        assert cache.head_index[0].tolist() == ctor["head_index"], case["name"]
+        assert cache.circular_cache_head_index[0].tolist() == ctor["circular_head"], case["name"]
+        assert cache.circular_cache_size[0].tolist() == ctor["circular_size"], case["name"]
+        assert cache.cache_update_index[0].tolist() == ctor["update_index"], case["name"]
         am = None
         if case["use_mask"]:
             am = torch.zeros(B, S, dtype=torch.int64, device=dev)

@@ -1,0 +1,96 @@
+"""The PRODUCT's copies of the plan -> cache-size rule and of the cache constructor
+(moa_amd.attention.cache_utils), on the CPU, against the vectors the reference's own code wrote
+(tests/golden/cache_update_vectors.json; made by tests/golden/make_cache_vectors.py) and against the
+oracle's copies.  Neither needs a GPU: the rule is host arithmetic and the constructor only lays out
+index tensors (reference: MoA/attention/cache_utils.py:1183-1239 and :698-769)."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from moa_amd.attention.cache_utils import StaticCircularCache, moa_config_to_cache_config
+from oracle import moa_oracle
+
+
+@pytest.fixture(scope="module")
+def golden(golden_dir):
+    return json.load(open(os.path.join(golden_dir, "cache_update_vectors.json")))
+
+
+def test_plan_rule_single_heads(golden):
+    rows = [p for p in golden["plans"] if "alpha" in p]
+    assert len(rows) == 7
+    for p in rows:
+        plan = {"alphas": [[p["alpha"]]], "betas": [[p["beta"]]]}
+        r = moa_config_to_cache_config(plan, p["seq_len"], p["max_new_token"], verbose=False)
+        assert r == {"cache_size": [[p["cache_size"]]], "static_size": [[p["static_size"]]]}, p
+        assert r == moa_oracle.moa_config_to_cache_config(plan, p["seq_len"], p["max_new_token"])
+
+
+def _check_rows(plan, rows):
+    for p in rows:
+        r = moa_config_to_cache_config(plan, p["seq_len"], p["max_new_token"], verbose=False)
+        assert r["cache_size"][0] == p["cache_size_layer0"]
+        assert r["cache_size"][-1] == p["cache_size_last"]
+        assert int(np.sum(r["cache_size"])) == p["cache_size_sum"]
+        assert int(np.sum(r["static_size"])) == p["static_size_sum"]
+        assert r == moa_oracle.moa_config_to_cache_config(plan, p["seq_len"], p["max_new_token"])
+
+
+def test_plan_rule_shipped_vicuna_7b(golden, golden_dir):
+    plan = json.load(open(os.path.join(golden_dir, "plan_vicuna-7b-v1.5-16k_moa_alpha_beta.json")))
+    rows = [p for p in golden["plans"] if p.get("plan_file", "").startswith("examples/lmsys--vicuna-7b")]
+    assert len(rows) == 2
+    _check_rows(plan, rows)
+
+
+def test_plan_rule_shipped_llama3_70b(golden):
+    """examples/gradientai--Llama-3-70B-Instruct-262k/streamingllm_alpha_beta.json of the reference is
+    80 layers x 64 heads of alpha = 0, beta = 0.5 (a uniform plan, written out here instead of copied)."""
+    plan = {"alphas": [[0.0] * 64 for _ in range(80)], "betas": [[0.5] * 64 for _ in range(80)]}
+    rows = [p for p in golden["plans"] if "Llama-3-70B" in p.get("plan_file", "")]
+    assert len(rows) == 2
+    _check_rows(plan, rows)
+
+
+def test_plan_rule_options():
+    """minimum_cache_size is applied after the clamp to the sequence (a cache may exceed it), sizes are
+    rounded up to split_size, sink_size caps the static part (reference :1224-1237)."""
+    plan = {"alphas": [[0, 1000, 5]], "betas": [[0.0, 0.0, 0.01]]}
+    r = moa_config_to_cache_config(plan, 100, 28, sink_size=96, minimum_cache_size=80, split_size=32, verbose=False)
+    assert r == {"cache_size": [[96, 128, 96]], "static_size": [[96, 96, 96]]}
+    assert r == moa_oracle.moa_config_to_cache_config(plan, 100, 28, sink_size=96, minimum_cache_size=80,
+                                                      split_size=32)
+
+
+def test_constructor_against_reference_vectors(golden):
+    for case in golden["cases"]:
+        B = case["B"]
+        c = StaticCircularCache([case["cache_size"]], static_size=[case["static_size"]], batch_size=B,
+                                head_dim=case["D"], device="cpu", dtype=torch.float32)
+        ctor, tag = case["ctor"], case["name"]
+        assert c.cache_head_start_index[0].tolist() == ctor["head_start"], tag
+        assert c.head_index[0].tolist() == ctor["head_index"], tag
+        assert c.circular_cache_head_index[0].tolist() == ctor["circular_head"], tag
+        assert c.circular_cache_size[0].tolist() == ctor["circular_size"], tag
+        assert c.cache_update_index[0].tolist() == ctor["update_index"], tag
+        assert c.cache_max_length[0].tolist() == case["cache_size"], tag
+        assert c.static_cache_size[0].tolist() == case["static_size"], tag
+        assert c.cache_valid_length[0].tolist() == [[0] * len(case["cache_size"])] * B, tag
+        assert c.mask_cache[0].shape == (B, sum(case["cache_size"])) and not c.mask_cache[0].any(), tag
+        for t in (c.cache_head_start_index[0], c.cache_update_index[0], c.cache_valid_length[0], c.mask_cache[0]):
+            assert t.dtype == torch.int64 and t.is_contiguous(), tag
+        assert len(c) == 1 and c.get_seq_length(0) == 0
+
+
+def test_constructor_several_layers_and_default_static():
+    c = StaticCircularCache([[128, 64], [64, 192, 64]], batch_size=2, head_dim=64)
+    assert len(c) == 2 and c.dtype == torch.float16
+    assert c.static_cache_size[1].tolist() == [0, 0, 0]
+    assert c.circular_cache_size[1].tolist() == [64, 192, 64]
+    assert c.head_index[1].tolist() == [0, 64, 256, 320]
+    assert c.layer_cache_size == [192, 320]
+    with pytest.raises(AssertionError):
+        StaticCircularCache([[64]], static_size=[[65]])
