@@ -68,6 +68,7 @@ class StaticCircularCache:
             c - s for c, s in zip(self.cache_max_length, self.static_cache_size)]
         self.layer_cache_size: List[int] = [sum(c) for c in cache_size]
         self._max_cache_size: List[int] = [max(c) for c in cache_size]
+        self._max_static_size: List[int] = [max(x) for x in static_size]
 
         starts = []
         for c in cache_size:
@@ -154,6 +155,20 @@ class StaticCircularCache:
             self.key_cache[layer_idx] = torch.zeros(shape, dtype=self.dtype, device=device)
             self.value_cache[layer_idx] = torch.zeros(shape, dtype=self.dtype, device=device)
 
+    def _check_capture(self, layer_idx: int, device) -> None:
+        """A decode step recorded into a HIP graph bakes in the host value ``kv_len``, which the
+        append kernels use for one decision only: has this head left its static part (the reference's
+        ``kv_len + 1 > static_size``, cache_utils.py:1041-1045).  A replay is right as long as that
+        decision does not change any more, i.e. once every head of the layer is past its sinks.
+        Capturing earlier would let replays walk a head's pointer linearly out of its segment.
+        (Replays do not advance ``get_seq_length()`` / ``cache_position`` either: callers that replay
+        pass explicit positions.)"""
+        if torch.cuda.is_current_stream_capturing() and self._kv_len[layer_idx] + 1 <= self._max_static_size[layer_idx]:
+            raise RuntimeError(
+                f"StaticCircularCache: layer {layer_idx} has seen {self._kv_len[layer_idx]} tokens, not more than its "
+                f"largest static size {self._max_static_size[layer_idx]}: a decode step captured now would be "
+                "replayed with the wrong ring decision; capture after the prompt has filled the static parts")
+
     def rope_update(
         self,
         query_states: Tensor,
@@ -197,6 +212,7 @@ class StaticCircularCache:
         self._to_device(layer_idx, device)
         if layer_idx == 0:
             self.cache_position += 1
+        self._check_capture(layer_idx, device)
         cos, sin, css = _cos_sin_strides(cos, sin, B, 1, D)
         qn, kn, vn = (t[:, :, -1, :] for t in (query_states, key_states, value_states))
         qn, kn, vn = (t if t.stride(-1) == 1 else t.contiguous() for t in (qn, kn, vn))
@@ -274,6 +290,7 @@ class StaticCircularCache:
         assert upd.is_contiguous() and self.cache_valid_length[layer_idx].is_contiguous()
 
         if seq_len == 1:
+            self._check_capture(layer_idx, device)
             kn = vn = None
             kns = vns = None
             if self.update_cache_content:

@@ -101,8 +101,11 @@ struct DecInt {
 // Chunk table of one batch row: prefix[h] = number of chunks of heads < h.
 // Built by all threads of the block (one thread per head: kDecThreads >= kMaxHeads): a shuffle
 // scan inside each wave, then the wave totals through LDS.  Returns the row's total chunk count.
+// Every entry is clamped to `cap`, the partial slots a batch row owns: with disjoint segments the clamp
+// never acts; with overlapping ones (lengths that sum to more than the row holds) the chunks past the cap
+// do not exist for any kernel that builds the table, so none of them is written, read or merged.
 template <int CHUNK, int NWAVES = kDecWaves>
-__device__ __forceinline__ int build_prefix(const int64_t* __restrict__ valid_row, int H,
+__device__ __forceinline__ int build_prefix(const int64_t* __restrict__ valid_row, int H, int cap,
                                             int* __restrict__ s_prefix /* [kMaxHeads + 1] */) {
   __shared__ int s_wave_total[NWAVES];
   const int tid = threadIdx.x;
@@ -124,7 +127,7 @@ __device__ __forceinline__ int build_prefix(const int64_t* __restrict__ valid_ro
   int base = 0;
 #pragma unroll
   for (int w = 0; w < NWAVES; ++w) base += (w < wave) ? s_wave_total[w] : 0;
-  if (tid < kMaxHeads) s_prefix[tid + 1] = base + incl;
+  if (tid < kMaxHeads) s_prefix[tid + 1] = min(base + incl, cap);
   if (tid == 0) s_prefix[0] = 0;
   __syncthreads();
   return s_prefix[H];
@@ -170,9 +173,9 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(
   const int col = lane % LPR;   // which 8-element slice of the row
   const int sub = lane / LPR;   // which row of a wave-wide load
 
-  // Disjoint segments give at most `cap` chunks per row; the clamp keeps partial
+  // Disjoint segments give at most `cap` chunks per row; the clamp inside keeps partial
   // slots inside the workspace if a caller hands in overlapping segments.
-  const int total = min(build_prefix<CHUNK>(head_valid + (int64_t)b * H, H, s_prefix), cap);
+  const int total = build_prefix<CHUNK>(head_valid + (int64_t)b * H, H, cap, s_prefix);
 
   for (int w = blockIdx.x; w < total; w += gridDim.x) {
     const int h = find_head(s_prefix, H, w);
@@ -354,7 +357,7 @@ __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
   __shared__ int s_n[GROUPS];
   const int b = blockIdx.y;
   const int tid = threadIdx.x;
-  build_prefix<CHUNK>(head_valid + (int64_t)b * H, H, s_prefix);
+  build_prefix<CHUNK>(head_valid + (int64_t)b * H, H, cap, s_prefix);
   const int grp = tid / D;
   const int d = tid % D;
   // every group runs the same number of rounds so that the barriers below are uniform
@@ -520,7 +523,7 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
     for (int dt = 0; dt < DT; ++dt) v_ad[dt] = ring0 + TILE_B + (v_rd ^ (uint32_t)(64 * dt));
   }
 
-  const int total = min(build_prefix<kGqaChunk, kGqaWaves>(head_valid + (int64_t)b * H, H, s_prefix), cap);
+  const int total = build_prefix<kGqaChunk, kGqaWaves>(head_valid + (int64_t)b * H, H, cap, s_prefix);
 
   for (int w = blockIdx.x; w < total; w += gridDim.x) {
     const int h = find_head(s_prefix, H, w);

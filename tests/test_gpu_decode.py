@@ -341,6 +341,43 @@ def test_maximum_head_count(dev):
         mixture_of_sparse_attention(q2, k2, k2, 0.125, head_start_index=hs2, head_valid_length=hv2)
 
 
+@pytest.mark.parametrize("G", [1, 4])
+def test_overlapping_segments_stay_defined(dev, G):
+    """Valid lengths that exceed the rings (what the cache's bookkeeping holds after a second prompt
+    insert, as in the reference: cache_utils.py:1136-1138 does not clamp): the segments overlap, a batch
+    row has more chunks than partial slots, and the chunk table is cut at the slot count in every kernel
+    alike.  Every output element must be written and finite; heads in front of the cut are exact."""
+    from moa_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(77 + G)
+    B, H, D, C = 2, 4, 128, 256
+    sumC = H * C
+    dtype = torch.float16
+    kc = torch.from_numpy(rng.standard_normal((B, sumC, D)).astype(np.float32)).to(dev, dtype)
+    vc = torch.from_numpy(rng.standard_normal((B, sumC, D)).astype(np.float32)).to(dev, dtype)
+    q = torch.from_numpy(rng.standard_normal((B, H * G, D)).astype(np.float32)).to(dev, dtype)
+    hs = np.broadcast_to(np.arange(H) * C, (B, H)).astype(np.int64).copy()
+    hv = (sumC - hs).astype(np.int64)                      # every head runs to the end of the row
+    hv[1, 0] = 5 * sumC                                    # and one far beyond it
+    o = torch.full((B, H * G, D), float("nan"), dtype=dtype, device=dev)
+    need = lib.moa_decode_workspace_bytes(B, H * G, H, D, sumC)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    hs_d, hv_d = torch.from_numpy(hs).to(dev), torch.from_numpy(hv).to(dev)
+    rc = lib.moa_decode_fwd(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), o.data_ptr(), ws.data_ptr(), ws.numel(),
+                            hs_d.data_ptr(), hv_d.data_ptr(), B, H * G, H, D, sumC, D ** -0.5,
+                            _lib.dtype_code(dtype), _lib.current_stream_ptr(dev))
+    assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all()
+    # head 0 of batch row 0 spans the whole row and lies in front of the cut for every chunk length
+    hv_clamped = np.minimum(hv, sumC - hs)
+    name = None if G == 1 else "f16"
+    ref = decode_segments(q.float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(), hs,
+                          hv_clamped, D ** -0.5, group=G, p_dtype=name)
+    err = np.abs(o[0, :G].float().cpu().numpy() - ref[0, :G])
+    assert (err <= ATOL + RTOL * np.abs(ref[0, :G])).all(), float(err.max())
+
+
 def test_errors(dev):
     from moa_amd import mixture_of_sparse_attention
     q = torch.zeros(1, 2, 1, 128, dtype=torch.float32, device=dev)

@@ -94,3 +94,20 @@ def test_constructor_several_layers_and_default_static():
     assert c.layer_cache_size == [192, 320]
     with pytest.raises(AssertionError):
         StaticCircularCache([[64]], static_size=[[65]])
+
+
+def test_capturing_a_decode_step_too_early_is_refused(monkeypatch):
+    """A decode step recorded into a graph bakes in kv_len, which decides whether a head has left its
+    static part: capture is only allowed once every head has (host logic, checked without a GPU)."""
+    c = StaticCircularCache([[128, 192]], static_size=[[64, 32]], batch_size=1, head_dim=64)
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: True)
+    for kv_len, ok in ((0, False), (40, False), (63, False), (64, True), (500, True)):
+        c._kv_len[0] = kv_len
+        if ok:
+            c._check_capture(0, "cpu")
+        else:
+            with pytest.raises(RuntimeError, match="static"):
+                c._check_capture(0, "cpu")
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: False)
+    c._kv_len[0] = 0
+    c._check_capture(0, "cpu")
