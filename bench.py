@@ -273,6 +273,8 @@ def bench_e2e(torch, dev, args, new_tokens=32):
     model = LlamaMixtureAttentionStack(L, hidden, Hq, num_key_value_heads=H, head_dim=D, dtype=dtype, device=dev)
     for p in model.parameters():
         p.data.normal_(0.0, hidden ** -0.5)
+    for layer in model.layers:       # the stack has no norms: small output projections keep the residual stream O(1)
+        layer.o_proj.weight.data.mul_(L ** -0.5)
     # a plan whose cache sizes are sink (64) + the elastic window at n_ctx
     if plan is None:
         plan = {"alphas": [[64 + s for s in elastic_spans(H, n_ctx, seed=l)] for l in range(L)],
