@@ -142,6 +142,26 @@ def bench_decode(torch, dev, args):
     torch.cuda.synchronize(dev)
     wall = time.perf_counter() - t0
 
+    # the same step with the rotary embedding of q and k folded into the append launch
+    # (StaticCircularCache.rope_update: what a caller that owns the projections runs)
+    ang = torch.rand(1, 1, D, generator=gen, device=dev) * 6.28
+    cos, sin = ang.cos().to(dtype), ang.sin().to(dtype)
+
+    def fused_step():
+        for l in range(L):
+            c = l % distinct
+            qe, kc, vc = cache.rope_update(qs[l], kn[l], vn[l], cos, sin, c)
+            mixture_of_sparse_attention(qe, kc, vc, sm, head_start_index=cache.cache_head_start_index[c],
+                                        head_valid_length=cache.cache_valid_length[c])
+
+    fused_step()
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        fused_step()
+    torch.cuda.synchronize(dev)
+    fused_wall = time.perf_counter() - t0
+
     app_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in events) / len(events)
     dec_ms = sum(e1.elapsed_time(e2) for _, e1, e2 in events) / len(events)
     rows_per_layer = rows_total / distinct
@@ -151,6 +171,9 @@ def bench_decode(torch, dev, args):
         "wall_s": wall,
         "tokens_per_s": B * args.steps / wall,
         "ms_per_step": wall / args.steps * 1e3,
+        "fused_rotary_step": {"workload": "the same step with the rotary embedding of q and k fused into the append launch",
+                              "ms_per_step": fused_wall / args.steps * 1e3,
+                              "tokens_per_s": B * args.steps / fused_wall},
         "decode_ms": dec_ms,
         "decode_bytes": dec_bytes,
         "decode_gbs": dec_bytes / (dec_ms * 1e-3) / 1e9,
@@ -203,10 +226,14 @@ def bench_rope_append(torch, dev, args, cache, iters=50):
             "GB/s": nbytes / (fused_us * 1e-6) / 1e9}
 
 
+C5_ALPHA_RANGE = (256.0, 8192.0)   # the largest config draws alpha from [256, 8192] (the others from [64, 2048])
+
+
 def bench_decode_gqa(torch, dev, args, iters=5, layers=8):
     """Decode attention at the grouped-query shape of the largest config (B=4, 64 query heads on 8
-    rings of head_dim 128, bf16, 32k context: 64 sinks + elastic window per ring): the matrix-core
-    kernel.  K+V bytes of the valid rows per launch over the mean HIP-event time around the call."""
+    rings of head_dim 128, bf16, 32k context: 64 sinks + elastic window per ring, alpha in
+    [256, 8192]): the matrix-core kernel.  K+V bytes of the valid rows per launch over the mean
+    HIP-event time around the call."""
     import numpy as np
     from moa_amd import mixture_of_sparse_attention
     from moa_amd.workloads import elastic_spans, ring_cache_sizes
@@ -215,7 +242,7 @@ def bench_decode_gqa(torch, dev, args, iters=5, layers=8):
         Hkv, G, D, ctx = 8, 8, 128, 32768
         caches = []
         for l in range(layers):
-            sizes, _ = ring_cache_sizes(elastic_spans(Hkv, ctx, seed=l))
+            sizes, _ = ring_cache_sizes(elastic_spans(Hkv, ctx, seed=l, alpha_range=C5_ALPHA_RANGE))
             sizes = np.asarray(sizes)
             sumc = int(sizes.sum())
             kc = torch.randn(B, sumc, D, device=dev, dtype=torch.bfloat16)
@@ -244,7 +271,8 @@ def bench_decode_gqa(torch, dev, args, iters=5, layers=8):
                         "frac_of_hbm_peak": byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
         del caches
         torch.cuda.empty_cache()
-    out["workload"] = "decode attention, 64 query heads on 8 rings, D=128, bf16, 32k context"
+    out["workload"] = ("decode attention, 64 query heads on 8 rings, D=128, bf16, 32k context, ring = 64 sinks + elastic "
+                       "window (alpha U[256,8192], beta U[0,0.5])")
     return out
 
 
@@ -401,16 +429,17 @@ def bench_e2e_full(torch, dev, args):
             "graph_decode_ms_per_step": graph_s * 1e3, "graph_decode_tokens_per_s": batch / graph_s}
 
 
-def bench_prefill(torch, dev, args, B=4, Hq=32, Hkv=32, N=8192, iters=None):
+def bench_prefill(torch, dev, args, B=4, Hq=32, Hkv=32, N=8192, iters=None, alpha_range=(64.0, 2048.0)):
     """One sparse prefill layer: the headline shape (B=4, 32 heads, N=8192) by default; the grouped-
-    query shape of the largest config with Hq=64, Hkv=8, N=32768 (spans per kv head)."""
+    query shape of the largest config with Hq=64, Hkv=8, N=32768 (spans per kv head, alpha in
+    [256, 8192])."""
     from moa_amd import mixture_of_sparse_attention
     from moa_amd.workloads import elastic_spans, prefill_work
 
     D = 128
     H = Hkv
     dtype = torch.bfloat16
-    spans = elastic_spans(H, N, seed=0)
+    spans = elastic_spans(H, N, seed=0, alpha_range=alpha_range)
     sink = torch.full((H,), 64, dtype=torch.int64, device=dev)
     local = torch.tensor(spans, dtype=torch.int64, device=dev)
     gen = torch.Generator(device=dev).manual_seed(7)
@@ -434,7 +463,8 @@ def bench_prefill(torch, dev, args, B=4, Hq=32, Hkv=32, N=8192, iters=None):
     ms = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
     med = ms[len(ms) // 2]
     return {
-        "workload": f"B={B},Hq={Hq},Hkv={Hkv},D=128,N={N},bf16,sink=64,window=elastic(seed 0)",
+        "workload": f"B={B},Hq={Hq},Hkv={Hkv},D=128,N={N},bf16,sink=64,window=elastic(seed 0, alpha "
+                    f"U[{alpha_range[0]:g},{alpha_range[1]:g}], beta U[0,0.5])",
         "ms_per_layer": med,
         "ms_min": ms[0],
         "flops_live": flops,
@@ -444,6 +474,31 @@ def bench_prefill(torch, dev, args, B=4, Hq=32, Hkv=32, N=8192, iters=None):
         "mfma_frac": flops / (med * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS,
         "mfma_peak_tflops": MFMA_PEAK_TFLOPS,
     }
+
+
+def bench_prefill_c1(torch, dev, iters=20):
+    """The CPU-reference configuration on the GPU kernel (fp16: the kernel has no fp32 path), to put a
+    GPU time beside cpu_baseline.prefill_c1."""
+    from moa_amd import mixture_of_sparse_attention
+    from moa_amd.workloads import uniform_block_windows
+    B, H, N, D = 1, 32, 2048, 64
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(B, N, H, D, generator=g).to(dev, torch.float16).transpose(1, 2) for _ in range(3))
+    sink = torch.full((H,), 64, dtype=torch.int64, device=dev)
+    local = torch.tensor(uniform_block_windows(H, seed=0), dtype=torch.int64, device=dev)
+    for _ in range(3):
+        mixture_of_sparse_attention(q, k, v, D ** -0.5, sink_size=sink, local_size=local)
+    torch.cuda.synchronize(dev)
+    evs = []
+    for _ in range(iters):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        mixture_of_sparse_attention(q, k, v, D ** -0.5, sink_size=sink, local_size=local)
+        e1.record()
+        evs.append((e0, e1))
+    torch.cuda.synchronize(dev)
+    ms = sorted(a.elapsed_time(b) for a, b in evs)
+    return {"workload": "B=1,H=32,D=64,N=2048,fp16,sink=64,window uniform in {256..1024}", "ms": ms[len(ms) // 2]}
 
 
 def cpu_baseline(torch, args, budget_s=12.0):
@@ -479,6 +534,8 @@ def cpu_baseline(torch, args, budget_s=12.0):
     # one token of ONE sequence costs L layer passes; the batch is B such sequences
     tok_s = 1.0 / (mean_layer * L)
     return {
+        "prefill_c1": cpu_prefill_c1(torch),
+        "append": cpu_append(torch, args),
         "value": tok_s,
         "unit": "tokens/s",
         "cores": threads,
@@ -486,6 +543,53 @@ def cpu_baseline(torch, args, budget_s=12.0):
         "sample": f"{len(per_layer)} (batch row, layer) decode passes of the same spans ({spent:.1f} s of CPU time), fp32 "
                   f"grouped SDPA on CPU; tokens/s = 1 / (mean pass time * {L} layers)",
     }
+
+
+def cpu_prefill_c1(torch):
+    """The CPU-reference configuration in full: one layer, B=1, 32 heads, head_dim 64, N=2048, fp32,
+    64 sinks + a window from {256,...,1024} per head, through the oracle's dense masked attention
+    (torch SDPA with a boolean mask, the arithmetic of the reference's dense path)."""
+    from oracle.moa_oracle import count_live_pairs, prefill_masked_dense
+    from moa_amd.workloads import uniform_block_windows
+    B, H, N, D = 1, 32, 2048, 64
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(B, H, N, D, generator=g) for _ in range(3))
+    ns, nl = [1] * H, [w // 64 for w in uniform_block_windows(H, seed=0)]
+    prefill_masked_dense(q[:, :2], k[:, :2], v[:, :2], D ** -0.5, ns[:2], nl[:2])   # warm-up
+    t0 = time.perf_counter()
+    prefill_masked_dense(q, k, v, D ** -0.5, ns, nl)
+    dt = time.perf_counter() - t0
+    pairs = sum(count_live_pairs(N, a, b)[0] for a, b in zip(ns, nl))
+    return {"seconds": dt, "cores": torch.get_num_threads(), "kind": "port",
+            "workload": "B=1,H=32,D=64,N=2048,fp32,sink=64,window uniform in {256..1024}: dense masked SDPA, whole config",
+            "gflops_live": 4.0 * D * pairs * B / dt / 1e9,
+            "gflops_dense_causal": 4.0 * D * H * B * (N * (N + 1) / 2) / dt / 1e9}
+
+
+def cpu_append(torch, args, rows=8, steps=20):
+    """The reference's decode-branch cache update (about 15 indexing operations per layer and step,
+    MoA/attention/cache_utils.py:1020-1058) as the oracle restates it with numpy, on `rows` batch rows
+    of one layer of the headline shape; the time of a whole batch is that times batch / rows (the work
+    is per batch row)."""
+    import numpy as np
+    from oracle.moa_oracle import StaticCircularCacheOracle
+    from moa_amd.workloads import elastic_spans, ring_cache_sizes
+    H, D = 32, 128
+    cs, ss = ring_cache_sizes(elastic_spans(H, args.ctx, seed=0))
+    o = StaticCircularCacheOracle(cs, ss, rows, D, dtype=np.float16)
+    o.cache_valid_length[:] = np.asarray(cs)[None, :]
+    o.cache_update_index[:] = o.circular_cache_head_index[None, :]
+    o.kv_len = args.ctx
+    rng = np.random.default_rng(0)
+    kn = rng.standard_normal((rows, H, 1, D)).astype(np.float16)
+    o.update_decode(kn, kn)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        o.update_decode(kn, kn)
+    dt = (time.perf_counter() - t0) / steps
+    return {"us_per_layer_step": dt * 1e6 * args.batch / rows, "cores": 1, "kind": "port",
+            "sample": f"{steps} decode-branch updates of {rows} batch rows of one layer (H=32, D=128, fp16, ctx "
+                      f"{args.ctx}), numpy index operations; scaled by {args.batch}/{rows} to the whole batch"}
 
 
 def main():
@@ -538,7 +642,9 @@ def main():
     if not args.no_prefill:
         try:
             pre = bench_prefill(torch, dev, args)
-            pre["grouped_query_32k"] = bench_prefill(torch, dev, args, B=1, Hq=64, Hkv=8, N=32768, iters=5)
+            pre["cpu_reference_config"] = bench_prefill_c1(torch, dev)
+            pre["grouped_query_32k"] = bench_prefill(torch, dev, args, B=1, Hq=64, Hkv=8, N=32768, iters=5,
+                                                     alpha_range=C5_ALPHA_RANGE)
         except NotImplementedError as e:
             pre = {"error": str(e)}
     torch.cuda.empty_cache()
@@ -581,6 +687,7 @@ def main():
         },
         "cpu_baseline": cpu,
         "append": {"us": dec["append_us"], "bytes": dec["append_bytes"], "GB/s": dec["append_gbs"]},
+        "fused_rotary_step": dec["fused_rotary_step"],
         "rope_append": rope,
         "prefill": pre,
         "decode_gqa": gqa,
