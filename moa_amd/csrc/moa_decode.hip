@@ -444,7 +444,10 @@ __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
 #ifndef MOA_GQA_BLOCKS
 #define MOA_GQA_BLOCKS 4
 #endif
-constexpr int kGqaChunk = MOA_GQA_CHUNK;   // cache rows per work-group step (a quarter per wave)
+// Cache rows per work-group step (a quarter per wave).  A chunk start costs a wave full memory
+// latencies with nothing in flight, so long chunks win: 2048 is the best of 512..4096 at batch 64 and at
+// batch 4.
+constexpr int kGqaChunk = MOA_GQA_CHUNK;
 constexpr int kGqaTile = 32;      // keys per MFMA tile
 constexpr int kGqaMaxG = 8;       // query heads per ring the per-wave result buffers are sized for
 #ifndef MOA_GQA_WAVES
@@ -461,7 +464,7 @@ template <> struct MfmaElem<BF16> { typedef PBF16 type; };
 template <int D>
 constexpr size_t gqa_lds_bytes() { return (size_t)kGqaWaves * kGqaStages * 2 * kGqaTile * D * 2; }
 
-template <typename T, int D>
+template <typename T, int D, int CHUNK>
 __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     uint16_t* __restrict__ o, float* __restrict__ part_acc, float* __restrict__ part_ml,
@@ -479,8 +482,9 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
   constexpr int TILE_B = kGqaTile * ROW_B;      // bytes of one K or V tile
   constexpr int NCP = TILE_B / 1024;            // async copies per tile and tensor
   constexpr int STAGE_B = 2 * TILE_B;           // K tile, then V tile
-  constexpr int WCHUNK = kGqaChunk / kGqaWaves;
+  constexpr int WCHUNK = CHUNK / kGqaWaves;
   constexpr float kRescaleStep = 8.f;
+  static_assert(WCHUNK % kGqaTile == 0, "a wave's share of a chunk is whole tiles");
 
   extern __shared__ __attribute__((aligned(1024))) char s_mem[];
   __shared__ int s_prefix[kMaxHeads + 1];
@@ -523,7 +527,7 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
     for (int dt = 0; dt < DT; ++dt) v_ad[dt] = ring0 + TILE_B + (v_rd ^ (uint32_t)(64 * dt));
   }
 
-  const int total = build_prefix<kGqaChunk, kGqaWaves>(head_valid + (int64_t)b * H, H, cap, s_prefix);
+  const int total = build_prefix<CHUNK, kGqaWaves>(head_valid + (int64_t)b * H, H, cap, s_prefix);
 
   for (int w = blockIdx.x; w < total; w += gridDim.x) {
     const int h = find_head(s_prefix, H, w);
@@ -534,7 +538,7 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
     int64_t len = head_valid[bh];
     if (seg0 < 0 || seg0 >= sumC) len = 0;   // clamp the segment into the row so that a bad index cannot fault
     if (len > sumC - seg0) len = sumC - seg0;
-    const int64_t r_begin = (int64_t)c * kGqaChunk + (int64_t)wave * WCHUNK;
+    const int64_t r_begin = (int64_t)c * CHUNK + (int64_t)wave * WCHUNK;
     int64_t r_end = r_begin + WCHUNK;
     if (r_end > len) r_end = len;
     const int n_rows = __builtin_amdgcn_readfirstlane(r_end > r_begin ? (int)(r_end - r_begin) : 0);
@@ -762,29 +766,46 @@ static int launch_decode(const void* q, const void* kc, const void* vc, void* o,
 }
 
 
-template <typename T, int D>
-static int launch_decode_gqa(const void* q, const void* kc, const void* vc, void* o, float* part_acc,
-                             float* part_ml, const int64_t* head_start, const int64_t* head_valid, int B,
-                             int H, int G, int64_t sumC, float sm_scale, hipStream_t st) {
+template <typename T, int D, int CHUNK>
+static int launch_decode_gqa_chunk(const void* q, const void* kc, const void* vc, void* o, float* part_acc,
+                                   float* part_ml, const int64_t* head_start, const int64_t* head_valid, int B,
+                                   int H, int G, int64_t sumC, float sm_scale, hipStream_t st) {
   const int cap = (int)decode_cap(sumC, H);   // partial slots per batch row the workspace was sized for
-  const int64_t chunks = (sumC + kGqaChunk - 1) / kGqaChunk + H;   // at most this many steps per batch row
+  const int64_t chunks = (sumC + CHUNK - 1) / CHUNK + H;   // at most this many steps per batch row
   int bx = (int)((256 * MOA_GQA_BLOCKS + B - 1) / B);   // one work-group per CU at a time (its LDS ring fills the CU)
   if (bx > chunks) bx = (int)chunks;
   if (bx < 1) bx = 1;
   constexpr size_t lds = gqa_lds_bytes<D>();
   static bool lds_reserved[kMaxDevices] = {};   // per template instance
-  if (int rc = reserve_lds(reinterpret_cast<const void*>(&decode_gqa_kernel<T, D>), lds, lds_reserved, "moa_decode_fwd"))
+  if (int rc = reserve_lds(reinterpret_cast<const void*>(&decode_gqa_kernel<T, D, CHUNK>), lds, lds_reserved, "moa_decode_fwd"))
     return rc;
-  hipLaunchKernelGGL((decode_gqa_kernel<T, D>), dim3(bx, B), dim3(kGqaThreads), lds, st,
+  hipLaunchKernelGGL((decode_gqa_kernel<T, D, CHUNK>), dim3(bx, B), dim3(kGqaThreads), lds, st,
                      (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, (uint16_t*)o,
                      part_acc, part_ml, head_start, head_valid, H, G, sumC, mfma_softmax_scale(sm_scale), cap);
   int rc = check_launch("moa_decode_fwd(grouped split)");
   if (rc) return rc;
   constexpr int GROUPS = kDecThreads / D;
   int mx = (H * G + GROUPS - 1) / GROUPS;
-  hipLaunchKernelGGL((decode_merge_kernel<T, D, kGqaChunk>), dim3(mx, B), dim3(kDecThreads), 0, st,
+  hipLaunchKernelGGL((decode_merge_kernel<T, D, CHUNK>), dim3(mx, B), dim3(kDecThreads), 0, st,
                      (uint16_t*)o, part_acc, part_ml, head_valid, H, G, cap);
   return check_launch("moa_decode_fwd(merge)");
+}
+
+template <typename T, int D>
+static int launch_decode_gqa(const void* q, const void* kc, const void* vc, void* o, float* part_acc,
+                             float* part_ml, const int64_t* head_start, const int64_t* head_valid, int B,
+                             int H, int G, int64_t sumC, float sm_scale, hipStream_t st) {
+  // One chunk length for every launch.  Measured at batch 4 of the 70B shape (213 MB of rings, about one
+  // 2048-row chunk per CU): 49.8 us per call with 2048-row chunks, 53.3 with 1024, 62.3 with 512 -- a chunk
+  // start costs three dependent memory latencies (ring index, query rows, first tiles), which shorter
+  // chunks pay more often than they win in balance.
+#define MOA_GQA_CALL(CH) \
+  launch_decode_gqa_chunk<T, D, CH>(q, kc, vc, o, part_acc, part_ml, head_start, head_valid, B, H, G, sumC, sm_scale, st)
+#ifdef MOA_GQA_FORCE_CHUNK   // experiment builds
+  return MOA_GQA_CALL(MOA_GQA_FORCE_CHUNK);
+#endif
+  return MOA_GQA_CALL(kGqaChunk);
+#undef MOA_GQA_CALL
 }
 
 // Launches the decode kernels with their partials in `workspace` (at least

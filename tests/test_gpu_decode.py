@@ -242,17 +242,18 @@ def test_grouped_query_decode(dev, dtype, G, D):
         torch.testing.assert_close(out1[:, 0].float(), out[:, 0, g::G].float(), rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("B", [2, 48])            # a grid smaller and larger than the chip
 @pytest.mark.parametrize("G", [2, 8])
-def test_grouped_query_boundaries_and_invariants(dev, G):
+def test_grouped_query_boundaries_and_invariants(dev, G, B):
     """The matrix-core kernel's edges: valid lengths around its 32-key tile, a wave's share (512
     rows) and its 2048-row chunk; scores that keep raising the running max (keys grow along the
     ring); the order of the rows inside a ring does not matter; V == 1 gives O == 1."""
     from moa_amd import mixture_of_sparse_attention
     rng = np.random.default_rng(7 + G)
     D, dtype = 128, torch.float16
-    lens = [1, 31, 32, 33, 511, 512, 513, 2047, 2048, 2049, 4097, 100]
+    lens = [1, 31, 32, 33, 127, 128, 129, 255, 256, 257, 511, 512, 513, 1023, 1024, 1025, 2047, 2048, 2049, 4097, 100]
     sizes = [max(64, -(-n // 64) * 64) for n in lens]
-    B, Hkv = 2, len(sizes)
+    Hkv = len(sizes)
     _, kc, vc, hs, hv = _case(rng, B, sizes, D, dtype, dev)
     hv[:] = np.asarray(lens)[None, :]
     hv[1, 3] = 0
@@ -261,10 +262,12 @@ def test_grouped_query_boundaries_and_invariants(dev, G):
     q = torch.from_numpy(rng.standard_normal((B, Hkv * G, 1, D)).astype(np.float32) * 2).to(dev, dtype)
     hs_t, hv_t = torch.from_numpy(hs).to(dev), torch.from_numpy(hv).to(dev)
     out = mixture_of_sparse_attention(q, kc, vc, D ** -0.5, head_start_index=hs_t, head_valid_length=hv_t)
-    _close_grouped(out[:, 0], q[:, :, 0], kc, vc, hs, hv, D ** -0.5, G, ("gqa edges", G))
+    rows = [0, 1, B - 1]                                    # the CPU oracle on three batch rows
+    _close_grouped(out[rows, 0], q[rows][:, :, 0], kc[rows], vc[rows], hs[rows], hv[rows], D ** -0.5, G,
+                   ("gqa edges", G, B))
     # reverse the valid rows of every ring (K and V alike): same softmax, same output
     kc2, vc2 = kc.clone(), vc.clone()
-    for b in range(B):
+    for b in rows:
         for h in range(Hkv):
             s0, n = int(hs[b, h]), int(hv[b, h])
             kc2[b, s0:s0 + n] = kc[b, s0:s0 + n].flip(0)
