@@ -98,22 +98,34 @@ struct DecInt {
   static constexpr int value = N;
 };
 
-// Chunk table of one batch row: prefix[h] = number of chunks of heads < h.
+// Chunk table of one batch row: prefix[h] = number of chunks of heads < h, and every head's segment
+// (first row, length) clamped into the row, so that a bad index cannot fault and a work-group finds a
+// chunk's segment in LDS instead of behind another memory latency.
 // Built by all threads of the block (one thread per head: kDecThreads >= kMaxHeads): a shuffle
 // scan inside each wave, then the wave totals through LDS.  Returns the row's total chunk count.
 // Every entry is clamped to `cap`, the partial slots a batch row owns: with disjoint segments the clamp
 // never acts; with overlapping ones (lengths that sum to more than the row holds) the chunks past the cap
 // do not exist for any kernel that builds the table, so none of them is written, read or merged.
+struct HeadTable {
+  int prefix[kMaxHeads + 1];
+  int seg0[kMaxHeads];   // first cache row of the head's segment (rows per batch row fit 31 bits: checked on the host)
+  int len[kMaxHeads];    // valid rows, clamped to the end of the batch row
+};
+
 template <int CHUNK, int NWAVES = kDecWaves>
-__device__ __forceinline__ int build_prefix(const int64_t* __restrict__ valid_row, int H, int cap,
-                                            int* __restrict__ s_prefix /* [kMaxHeads + 1] */) {
+__device__ __forceinline__ int build_prefix(const int64_t* __restrict__ valid_row, const int64_t* __restrict__ start_row,
+                                            int H, int64_t sumC, int cap, HeadTable* __restrict__ tab) {
   __shared__ int s_wave_total[NWAVES];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   int n = 0;
   if (tid < H) {
     int64_t len = valid_row[tid];
-    if (len < 0) len = 0;
+    const int64_t seg0 = start_row[tid];
+    if (len < 0 || seg0 < 0 || seg0 >= sumC) len = 0;
+    if (len > sumC - seg0) len = sumC - seg0;
+    tab->seg0[tid] = (int)(len > 0 ? seg0 : 0);
+    tab->len[tid] = (int)len;
     n = (int)((len + CHUNK - 1) / CHUNK);
   }
   int incl = n;   // inclusive scan inside the wave
@@ -127,10 +139,10 @@ __device__ __forceinline__ int build_prefix(const int64_t* __restrict__ valid_ro
   int base = 0;
 #pragma unroll
   for (int w = 0; w < NWAVES; ++w) base += (w < wave) ? s_wave_total[w] : 0;
-  if (tid < kMaxHeads) s_prefix[tid + 1] = min(base + incl, cap);
-  if (tid == 0) s_prefix[0] = 0;
+  if (tid < kMaxHeads) tab->prefix[tid + 1] = min(base + incl, cap);
+  if (tid == 0) tab->prefix[0] = 0;
   __syncthreads();
-  return s_prefix[H];
+  return tab->prefix[H];
 }
 
 // Largest h with prefix[h] <= w  (w < prefix[H]).
@@ -161,7 +173,8 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(
   constexpr int WCHUNK = CHUNK / kDecWaves;
   static_assert(WCHUNK % ROWS == 0, "chunk must split evenly over waves and load batches");
 
-  __shared__ int s_prefix[kMaxHeads + 1];
+  __shared__ HeadTable s_tab;
+  const int* const s_prefix = s_tab.prefix;
   __shared__ float s_acc[kDecWaves][G][D];
   __shared__ float s_m[kDecWaves][G];
   __shared__ float s_l[kDecWaves][G];
@@ -175,18 +188,15 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(
 
   // Disjoint segments give at most `cap` chunks per row; the clamp inside keeps partial
   // slots inside the workspace if a caller hands in overlapping segments.
-  const int total = build_prefix<CHUNK>(head_valid + (int64_t)b * H, H, cap, s_prefix);
+  const int total = build_prefix<CHUNK>(head_valid + (int64_t)b * H, head_start + (int64_t)b * H, H, sumC, cap, &s_tab);
 
   for (int w = blockIdx.x; w < total; w += gridDim.x) {
     const int h = find_head(s_prefix, H, w);
     const int c = w - s_prefix[h];
     const int n_chunks = s_prefix[h + 1] - s_prefix[h];
     const int64_t bh = (int64_t)b * H + h;
-    const int64_t seg0 = head_start[bh];
-    int64_t len = head_valid[bh];
-    // clamp the segment into the row so that a bad index cannot fault
-    if (seg0 < 0 || seg0 >= sumC) len = 0;
-    if (len > sumC - seg0) len = sumC - seg0;
+    const int64_t seg0 = s_tab.seg0[h];
+    const int64_t len = s_tab.len[h];
     const int64_t r_begin = (int64_t)c * CHUNK + (int64_t)wave * WCHUNK;
     int64_t r_end = r_begin + WCHUNK;
     if (r_end > len) r_end = len;
@@ -349,15 +359,17 @@ __global__ __launch_bounds__(kDecThreads) void decode_split_kernel(
 template <typename T, int D, int CHUNK>
 __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
     uint16_t* __restrict__ o, const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-    const int64_t* __restrict__ head_valid, int H, int G /* query heads per ring */, int cap) {
+    const int64_t* __restrict__ head_start, const int64_t* __restrict__ head_valid, int H,
+    int G /* query heads per ring */, int64_t sumC, int cap) {
   constexpr int GROUPS = kDecThreads / D;
   constexpr int kFactors = 64;   // chunks whose factors are staged at a time
-  __shared__ int s_prefix[kMaxHeads + 1];
+  __shared__ HeadTable s_tab;
+  const int* const s_prefix = s_tab.prefix;
   __shared__ float s_f[GROUPS][kFactors];
   __shared__ int s_n[GROUPS];
   const int b = blockIdx.y;
   const int tid = threadIdx.x;
-  build_prefix<CHUNK>(head_valid + (int64_t)b * H, H, cap, s_prefix);
+  build_prefix<CHUNK>(head_valid + (int64_t)b * H, head_start + (int64_t)b * H, H, sumC, cap, &s_tab);
   const int grp = tid / D;
   const int d = tid % D;
   // every group runs the same number of rounds so that the barriers below are uniform
@@ -487,7 +499,8 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
   static_assert(WCHUNK % kGqaTile == 0, "a wave's share of a chunk is whole tiles");
 
   extern __shared__ __attribute__((aligned(1024))) char s_mem[];
-  __shared__ int s_prefix[kMaxHeads + 1];
+  __shared__ HeadTable s_tab;
+  const int* const s_prefix = s_tab.prefix;
   // the per-wave results (m, l, O[d] per query head) go into the first 4.5 KiB of the wave's own ring
   // once its loop is over
   __shared__ float s_m[kGqaWaves][kGqaMaxG];
@@ -527,17 +540,15 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
     for (int dt = 0; dt < DT; ++dt) v_ad[dt] = ring0 + TILE_B + (v_rd ^ (uint32_t)(64 * dt));
   }
 
-  const int total = build_prefix<CHUNK, kGqaWaves>(head_valid + (int64_t)b * H, H, cap, s_prefix);
+  const int total = build_prefix<CHUNK, kGqaWaves>(head_valid + (int64_t)b * H, head_start + (int64_t)b * H, H, sumC, cap, &s_tab);
 
   for (int w = blockIdx.x; w < total; w += gridDim.x) {
     const int h = find_head(s_prefix, H, w);
     const int c = w - s_prefix[h];
     const int n_chunks = s_prefix[h + 1] - s_prefix[h];
     const int64_t bh = (int64_t)b * H + h;
-    const int64_t seg0 = head_start[bh];
-    int64_t len = head_valid[bh];
-    if (seg0 < 0 || seg0 >= sumC) len = 0;   // clamp the segment into the row so that a bad index cannot fault
-    if (len > sumC - seg0) len = sumC - seg0;
+    const int64_t seg0 = s_tab.seg0[h];
+    const int64_t len = s_tab.len[h];
     const int64_t r_begin = (int64_t)c * CHUNK + (int64_t)wave * WCHUNK;
     int64_t r_end = r_begin + WCHUNK;
     if (r_end > len) r_end = len;
@@ -747,7 +758,7 @@ static int launch_decode(const void* q, const void* kc, const void* vc, void* o,
     int rc = check_launch("moa_decode_fwd(split)");
     if (rc) return rc;
     hipLaunchKernelGGL((decode_merge_kernel<T, D, kSmallChunk>), dim3(mx, B), dim3(kDecThreads), 0, st,
-                       (uint16_t*)o, part_acc, part_ml, head_valid, H, G, cap);
+                       (uint16_t*)o, part_acc, part_ml, head_start, head_valid, H, G, sumC, cap);
     return check_launch("moa_decode_fwd(merge)");
   }
   if (pipe)
@@ -761,7 +772,7 @@ static int launch_decode(const void* q, const void* kc, const void* vc, void* o,
   int rc = check_launch("moa_decode_fwd(split)");
   if (rc) return rc;
   hipLaunchKernelGGL((decode_merge_kernel<T, D, kChunk>), dim3(mx, B), dim3(kDecThreads), 0, st,
-                     (uint16_t*)o, part_acc, part_ml, head_valid, H, G, cap);
+                     (uint16_t*)o, part_acc, part_ml, head_start, head_valid, H, G, sumC, cap);
   return check_launch("moa_decode_fwd(merge)");
 }
 
@@ -787,7 +798,7 @@ static int launch_decode_gqa_chunk(const void* q, const void* kc, const void* vc
   constexpr int GROUPS = kDecThreads / D;
   int mx = (H * G + GROUPS - 1) / GROUPS;
   hipLaunchKernelGGL((decode_merge_kernel<T, D, CHUNK>), dim3(mx, B), dim3(kDecThreads), 0, st,
-                     (uint16_t*)o, part_acc, part_ml, head_valid, H, G, cap);
+                     (uint16_t*)o, part_acc, part_ml, head_start, head_valid, H, G, sumC, cap);
   return check_launch("moa_decode_fwd(merge)");
 }
 
@@ -838,6 +849,7 @@ static int decode_check_args(const char* who, const void* q, const void* kc, con
   if (!q || !kc || !vc || !o || !head_start || !head_valid_len) return fail(MOA_ERR_ARG, "%s: null pointer", who);
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || sumC <= 0) return fail(MOA_ERR_ARG, "%s: B, H, sumC must be positive", who);
   if (B > 65535) return fail(MOA_ERR_UNSUPPORTED, "%s: B <= 65535", who);
+  if (sumC >= ((int64_t)1 << 31)) return fail(MOA_ERR_UNSUPPORTED, "%s: at most 2^31 - 1 cache rows per batch row", who);
   if (Hq % Hkv != 0) return fail(MOA_ERR_ARG, "%s: Hq=%d is not a multiple of Hkv=%d", who, Hq, Hkv);
   const int G = Hq / Hkv;
   if (G > kGqaMaxG) return fail(MOA_ERR_UNSUPPORTED, "%s: %d query heads per kv head (at most %d)", who, G, kGqaMaxG);
