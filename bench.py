@@ -57,6 +57,10 @@ def parse_args():
                     help="with --only e2e: 7b = 32 layers, 32 heads, B=8, 16k prompt, fp16; 70b = 80 layers, 64 query "
                          "heads on 8 kv heads, hidden 8192, B=4, 32k prompt, bf16 (the largest config)")
     ap.add_argument("--new-tokens", type=int, default=64, help="with --only e2e-full: decode steps to time")
+    ap.add_argument("--test_mode", choices=["prefill", "decode", "whole"], default=None,
+                    help="run moa_amd.efficiency_test (the reference's efficiency script: same modes and printed "
+                         "figures) on the whole decoder of --shape at that config's batch and prompt length, "
+                         "--new-tokens decode steps; not the contract line")
     ap.add_argument("--only", choices=["decode", "prefill", "copy", "e2e", "e2e-full", "gqa"], default=None,
                     help="profiling aid: run one part only and print its figures (not the contract line)")
     return ap.parse_args()
@@ -621,6 +625,14 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.test_mode:
+        from moa_amd import efficiency_test
+        batch, prompt = (4, 32768) if args.shape == "70b" else (8, 16384)
+        efficiency_test.run_model(efficiency_test.parse_args(
+            ["--prefill_len", str(prompt), "--decode_len", str(args.new_tokens), "--batch_size", str(batch),
+             "--model_name", args.shape, "--dtype", "bf16", "--test_mode", args.test_mode, "--cuda_event", "--cuda_cache"]
+            + (["--moa_config", args.plan] if args.plan else [])))
+        return
     if args.only == "copy":
         # calibration for the HBM traffic counters: a plain device copy of known size (1 GiB read,
         # 1 GiB written per launch by torch's elementwise copy kernel)

@@ -394,11 +394,52 @@ def moa_config_to_cache_config(
         static_size.append(ss)
     if verbose:
         print("Cache configuration")
-        print(f"{'layer':>5} {'heads':>5} {'raw':>8} {'mean':>9} {'min':>7} {'max':>7} {'ratio':>6}")
-        for l, cs in enumerate(cache_size):
-            print(f"{l:>5} {len(cs):>5} {n_total:>8} {sum(cs) / len(cs):>9.1f} {min(cs):>7} {max(cs):>7} "
-                  f"{sum(cs) / len(cs) / n_total:>6.2f}")
-        flat = [c for cs in cache_size for c in cs]
-        print(f"model: mean {sum(flat) / len(flat):.1f} min {min(flat)} max {max(flat)} "
-              f"ratio {sum(flat) / len(flat) / n_total:.2f}")
+        print(format_cache_summary(*cache_config_summary(cache_size, static_size, n_total)))
     return {"cache_size": cache_size, "static_size": static_size}
+
+
+_SUMMARY_METRICS = ("cache_size", "static_size", "circular_size", "ratio")
+
+
+def cache_config_summary(cache_size, static_size, raw_cache_size):
+    """What the reference prints for a cache configuration (MoA/attention/cache_utils.py:1241-1293), as
+    data: per layer the mean raw size (``seq_len + max_new_token``) and the (mean, min, max) over heads
+    of cache_size, static_size, circular_size = cache - static and ratio = cache / raw; for the whole
+    model the same four metrics plus raw_cache_size over all heads.  Returns ``(layer_rows, model_rows)``:
+    ``layer_rows[l][metric] = (mean, min, max)`` and ``model_rows[metric] = (mean, min, max)``."""
+    def stats(xs):
+        return (sum(xs) / len(xs), min(xs), max(xs))
+
+    def metrics(cs, ss):
+        return {"cache_size": list(cs), "static_size": list(ss), "circular_size": [c - s for c, s in zip(cs, ss)],
+                "ratio": [c / raw_cache_size for c in cs]}
+
+    layer_rows = []
+    for cs, ss in zip(cache_size, static_size):
+        row = {k: stats(v) for k, v in metrics(cs, ss).items()}
+        row["raw_cache_size"] = (float(raw_cache_size),) * 3
+        layer_rows.append(row)
+    flat_c = [c for cs in cache_size for c in cs]
+    flat_s = [x for ss in static_size for x in ss]
+    model_rows = {k: stats(v) for k, v in metrics(flat_c, flat_s).items()}
+    model_rows["raw_cache_size"] = (float(raw_cache_size),) * 3
+    return layer_rows, model_rows
+
+
+def format_cache_summary(layer_rows, model_rows) -> str:
+    """The two tables of the reference's printout (per layer, then the model), two decimals like its
+    ``pd.options.display.float_format``; plain text, no pandas."""
+    head = f"{'layer_id':>8} {'raw_cache_size':>14}" + "".join(
+        f" {m + ' mean':>19} {'min':>9} {'max':>9}" for m in _SUMMARY_METRICS)
+    lines = [head]
+    for l, row in enumerate(layer_rows):
+        line = f"{l:>8} {row['raw_cache_size'][0]:>14.2f}"
+        for m in _SUMMARY_METRICS:
+            mean, lo, hi = row[m]
+            line += f" {mean:>19.2f} {lo:>9.2f} {hi:>9.2f}"
+        lines.append(line)
+    lines.append(f"{'metric':>16} {'max':>12} {'mean':>12} {'min':>12}")
+    for m in ("cache_size", "circular_size", "ratio", "raw_cache_size", "static_size"):
+        mean, lo, hi = model_rows[m]
+        lines.append(f"{m:>16} {hi:>12.2f} {mean:>12.2f} {lo:>12.2f}")
+    return "\n".join(lines)

@@ -35,6 +35,45 @@ def rotary_cos_sin(position_ids: Tensor, head_dim: int, dtype: torch.dtype, base
     return emb.cos().to(dtype), emb.sin().to(dtype)
 
 
+def attention_geometry(attn) -> Tuple[int, int, int]:
+    """(query heads, kv heads, head_dim) of an attention module: this package's LlamaMixtureAttention or
+    a transformers Llama attention (whose head counts live in its config)."""
+    cfg = getattr(attn, "config", None)
+    num_heads = getattr(attn, "num_heads", None) or cfg.num_attention_heads
+    num_kv = getattr(attn, "num_key_value_heads", None) or getattr(cfg, "num_key_value_heads", None) or num_heads
+    head_dim = getattr(attn, "head_dim", None) or attn.q_proj.out_features // num_heads
+    return int(num_heads), int(num_kv), int(head_dim)
+
+
+def mixture_attention_forward(attn, hidden_states: Tensor, position_embeddings: Tuple[Tensor, Tensor],
+                              past_key_value: StaticCircularCache, attention_mask: Optional[Tensor] = None) -> Tensor:
+    """The body of the reference's ``LlamaMixtureAttention.forward`` (modeling_llama.py:232-326) for any
+    module ``attn`` with ``q_proj / k_proj / v_proj / o_proj`` and a ``layer_idx``: projections, rotary
+    embedding + cache update (one launch in decode), sparse attention, output projection.
+    hidden_states ``[batch, q_len, hidden]``; position_embeddings ``(cos, sin)`` each
+    ``[batch or 1, q_len, head_dim]``; attention_mask ``[batch, kv_len]`` of 0/1 marks left padding of a
+    prompt.  Returns ``[batch, q_len, hidden]``."""
+    assert not attn.training, "only support inference now"
+    assert isinstance(past_key_value, StaticCircularCache)
+    num_heads, num_kv, head_dim = attention_geometry(attn)
+    bsz, q_len, _ = hidden_states.shape
+    # [B, q_len, H*D] viewed as [B, H, q_len, D]: no copy, the kernels take the strides
+    q = attn.q_proj(hidden_states).view(bsz, q_len, num_heads, head_dim).transpose(1, 2)
+    k = attn.k_proj(hidden_states).view(bsz, q_len, num_kv, head_dim).transpose(1, 2)
+    v = attn.v_proj(hidden_states).view(bsz, q_len, num_kv, head_dim).transpose(1, 2)
+    cos, sin = position_embeddings
+    li = attn.layer_idx
+    q, keys, values = past_key_value.rope_update(q, k, v, cos, sin, li, attention_mask)
+    out = mixture_of_sparse_attention(
+        q, keys, values, sm_scale=head_dim ** -0.5, attention_dropout=0.0,
+        sink_size=past_key_value.static_cache_size[li],
+        local_size=past_key_value.circular_cache_size[li],
+        head_start_index=past_key_value.cache_head_start_index[li],
+        head_valid_length=past_key_value.cache_valid_length[li],
+    )   # [batch, q_len, heads, head_dim]
+    return attn.o_proj(out.reshape(bsz, q_len, num_heads * head_dim))
+
+
 class LlamaMixtureAttention(nn.Module):
     """One attention layer.  ``forward`` follows the reference's (:232-326)."""
 
@@ -60,27 +99,10 @@ class LlamaMixtureAttention(nn.Module):
         """hidden_states ``[batch, q_len, hidden]``; position_embeddings ``(cos, sin)`` each
         ``[batch or 1, q_len, head_dim]``; attention_mask ``[batch, kv_len]`` of 0/1 marks left
         padding of a prompt.  Returns ``[batch, q_len, hidden]``."""
-        assert not self.training, "only support inference now"
-        assert isinstance(past_key_value, StaticCircularCache)
-        bsz, q_len, _ = hidden_states.shape
-        # [B, q_len, H*D] viewed as [B, H, q_len, D]: no copy, the kernels take the strides
-        q = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
-        k = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
-        v = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
-        cos, sin = position_embeddings
-        q, keys, values = past_key_value.rope_update(q, k, v, cos, sin, self.layer_idx, attention_mask)
-        li = self.layer_idx
-        attn = mixture_of_sparse_attention(
-            q, keys, values, sm_scale=self.head_dim ** -0.5, attention_dropout=0.0,
-            sink_size=past_key_value.static_cache_size[li],
-            local_size=past_key_value.circular_cache_size[li],
-            head_start_index=past_key_value.cache_head_start_index[li],
-            head_valid_length=past_key_value.cache_valid_length[li],
-        )   # [batch, q_len, heads, head_dim]
-        return self.o_proj(attn.reshape(bsz, q_len, self.num_heads * self.head_dim))
+        return mixture_attention_forward(self, hidden_states, position_embeddings, past_key_value, attention_mask)
 
 
-def install_plan(attention_layers: List["LlamaMixtureAttention"], moa_config: Dict, permute_head: bool) -> Dict:
+def install_plan(attention_layers: List[nn.Module], moa_config: Dict, permute_head: bool) -> Dict:
     """What ``set_mixture_of_attention`` does to the plan and the projections (reference :373-398):
     returns the plan as stored on the model (re-ordered like the heads when ``permute_head``)."""
     alphas = [list(a) for a in moa_config["alphas"]]
@@ -92,7 +114,8 @@ def install_plan(attention_layers: List["LlamaMixtureAttention"], moa_config: Di
             i = layer.layer_idx
             alphas[i] = [alphas[i][j] for j in perm.tolist()]
             betas[i] = [betas[i][j] for j in perm.tolist()]
-            hk, g = layer.num_key_value_heads, layer.num_key_value_groups
+            heads, hk, _ = attention_geometry(layer)
+            g = heads // hk
             permute_attention_projection(layer.q_proj, perm, hk, g)
             permute_attention_projection(layer.k_proj, perm, hk)
             permute_attention_projection(layer.v_proj, perm, hk)
@@ -276,3 +299,92 @@ class LlamaMixtureForCausalLM(nn.Module):
             out.append(nxt)
             logits, cache = self.forward(nxt, cache)
         return torch.cat(out, dim=1)
+
+
+# ---- binding the path into a transformers-style Llama model -------------------------------------------
+# The reference patches a loaded transformers model in place: update_model_function (MoA/models/interface.py)
+# binds set_mixture_of_attention to ``model.model``; calling it swaps in the model forward and the attention
+# forwards below (MoA/models/llama/modeling_llama.py:334-406).  The same here, for any model whose
+# ``model.model`` has ``embed_tokens``, ``layers[i].{input_layernorm, self_attn, post_attention_layernorm,
+# mlp}``, ``norm`` and a ``config`` (a transformers LlamaModel of any recent release: only submodule names
+# are relied on, not its internal mask and cache helpers, which changed between releases).
+
+
+def _rope_base(config) -> float:
+    params = getattr(config, "rope_parameters", None)
+    if isinstance(params, dict) and "rope_theta" in params:
+        kind = params.get("rope_type", "default")
+        if kind != "default":
+            raise NotImplementedError(f"rope_type {kind!r}: only the default rotary embedding is covered")
+        return float(params["rope_theta"])
+    if getattr(config, "rope_scaling", None):
+        raise NotImplementedError("rope_scaling: only the default rotary embedding is covered")
+    return float(getattr(config, "rope_theta", 10000.0))
+
+
+def LlamaModel_MixtureAttention_forward(self, input_ids=None, attention_mask=None, position_ids=None,
+                                        past_key_values=None, inputs_embeds=None, use_cache=None, **kwargs):
+    """Model forward with the MoA attention path (reference modeling_llama.py:52-204): builds the
+    StaticCircularCache from the plan at the first call of a generation (any other kind of cache passed
+    in is replaced, as in the reference :93-112), continues the positions from the cache, runs the
+    decoder layers with the attention of ``mixture_attention_forward``.  Returns an object with
+    ``last_hidden_state`` (only the last position when ``last_hidden_only`` was set, :188-190) and
+    ``past_key_values`` (the StaticCircularCache)."""
+    assert self.use_moa, "call set_mixture_of_attention first"
+    if (input_ids is None) == (inputs_embeds is None):
+        raise ValueError("You must specify exactly one of input_ids or inputs_embeds")
+    hidden_states = self.embed_tokens(input_ids) if inputs_embeds is None else inputs_embeds
+    bsz, q_len = hidden_states.shape[:2]
+    _, _, head_dim = attention_geometry(self.layers[0].self_attn)
+    if not isinstance(past_key_values, StaticCircularCache):
+        past_key_values = new_cache_for_plan(self.moa_config, self.moa_max_new_token, bsz, q_len, head_dim,
+                                             hidden_states.device, hidden_states.dtype)
+    if position_ids is None:
+        past = past_key_values.get_seq_length()
+        position_ids = torch.arange(past, past + q_len, device=hidden_states.device)[None, :]
+    if attention_mask is not None and not (attention_mask == 0).any():
+        attention_mask = None    # a mask without padding is no mask (:119-121)
+    cos_sin = rotary_cos_sin(position_ids, head_dim, hidden_states.dtype, _rope_base(self.config))
+    with torch.no_grad():
+        for layer in self.layers:
+            residual = hidden_states
+            hidden_states = residual + mixture_attention_forward(layer.self_attn, layer.input_layernorm(hidden_states),
+                                                                 cos_sin, past_key_values, attention_mask)
+            hidden_states = hidden_states + layer.mlp(layer.post_attention_layernorm(hidden_states))
+        hidden_states = self.norm(hidden_states)
+    if self.last_hidden_only:
+        hidden_states = hidden_states[:, -1:, :]
+    try:
+        from transformers.modeling_outputs import BaseModelOutputWithPast
+        return BaseModelOutputWithPast(last_hidden_state=hidden_states, past_key_values=past_key_values)
+    except ImportError:   # a duck-typed model without transformers installed
+        from types import SimpleNamespace
+        return SimpleNamespace(last_hidden_state=hidden_states, past_key_values=past_key_values,
+                               hidden_states=None, attentions=None)
+
+
+def LlamaModel_set_mixture_of_attention(self, moa_config: Dict, permute_head: bool = False, moa_verbose: bool = False,
+                                        moa_max_new_token: int = 1024, last_hidden_only: bool = True,
+                                        sparse_prefill: bool = True) -> None:
+    """Same arguments as the reference's function of this name (modeling_llama.py:334-406): stores the
+    plan, optionally clusters heads with equal (alpha, beta) by permuting the plan and the q/k/v/o
+    projections of every layer, and swaps in the MoA model forward."""
+    from types import MethodType
+
+    assert sparse_prefill, "only support sparse prefill now"
+    for i, layer in enumerate(self.layers):
+        if getattr(layer.self_attn, "layer_idx", None) is None:
+            layer.self_attn.layer_idx = i
+    plan = {"alphas": [list(a) for a in moa_config["alphas"]], "betas": [list(b) for b in moa_config["betas"]]}
+    self.moa_config = install_plan([layer.self_attn for layer in self.layers], plan, permute_head)
+    self.moa_verbose = moa_verbose
+    self.last_hidden_only = last_hidden_only
+    self.moa_max_new_token = moa_max_new_token
+    self.use_moa = True
+    self.forward = MethodType(LlamaModel_MixtureAttention_forward, self)
+    self.eval()
+
+
+def LlamaModel_use_block_sparse_attention_lut(self, *args, **kwargs):
+    """The reference's older lookup-table sparse attention (deprecated there); not part of this path."""
+    raise NotImplementedError("the lookup-table sparse attention is not part of this build; use set_mixture_of_attention")

@@ -111,3 +111,59 @@ def test_capturing_a_decode_step_too_early_is_refused(monkeypatch):
     monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: False)
     c._kv_len[0] = 0
     c._check_capture(0, "cpu")
+
+
+def test_update_model_function_binds_like_the_reference():
+    """Host logic of the wrapper binding (MoA/models/interface.py:3-28): Llama-family names get
+    set_mixture_of_attention bound to model.model, others raise; the plan is stored (and re-ordered with
+    the projections when heads are permuted)."""
+    from types import SimpleNamespace
+    from torch import nn
+    from moa_amd.models.interface import update_model_function
+    from moa_amd.models.llama.modeling_llama import LlamaMixtureAttention
+
+    layers = nn.ModuleList(nn.Module() for _ in range(2))
+    for i, l in enumerate(layers):
+        l.self_attn = LlamaMixtureAttention(64, 4, 2, head_dim=16, layer_idx=i, dtype=torch.float32)
+    inner = nn.Module()
+    inner.layers = layers
+    model = SimpleNamespace(model=inner)
+    with pytest.raises(NotImplementedError):
+        update_model_function(model, "gpt2")
+    assert update_model_function(model, "lmsys/longchat-7b") is model
+    w_before = layers[0].self_attn.k_proj.weight.data.clone()
+    inner.set_mixture_of_attention({"alphas": [[512.0, 128.0], [64.0, 64.0]], "betas": [[0.0, 0.0]] * 2},
+                                   permute_head=True, moa_max_new_token=16)
+    assert inner.use_moa and inner.moa_max_new_token == 16 and inner.last_hidden_only
+    assert inner.moa_config["alphas"] == [[128.0, 512.0], [64.0, 64.0]]          # layer 0: heads swapped
+    w_after = layers[0].self_attn.k_proj.weight.data
+    assert torch.equal(w_after.view(2, 16, 64)[0], w_before.view(2, 16, 64)[1])
+    assert torch.equal(layers[1].self_attn.k_proj.weight.data.view(2, 16, 64)[0],
+                       layers[1].self_attn.k_proj.weight.data.view(2, 16, 64)[0])
+    with pytest.raises(NotImplementedError):
+        inner.use_block_sparse_attention_lut()
+
+
+def test_efficiency_cli_arguments():
+    from moa_amd import efficiency_test
+    a = efficiency_test.parse_args(["--prefill_len", "4096"])
+    assert (a.test_mode, a.num_iters, a.batch_size, a.decode_len, a.model_name) == (
+        "whole", 1, 1, None, "lmsys/vicuna-7b-v1.5-16k")
+    assert efficiency_test.shape_of("lmsys/vicuna-7b-v1.5-16k")[0] == "7b"
+    assert efficiency_test.shape_of("lmsys/vicuna-13b-v1.5-16k")[1][:4] == (40, 5120, 40, 40)
+    assert efficiency_test.shape_of("gradientai/Llama-3-70B-Instruct-262k")[1][2:4] == (64, 8)
+    with pytest.raises(NotImplementedError):
+        efficiency_test.shape_of("gpt2")
+
+
+def test_cache_summary_columns():
+    """The reference's cache summary (MoA/attention/cache_utils.py:1241-1293): per layer and for the model,
+    (mean, min, max) of cache_size, static_size, circular_size and ratio = cache / (seq_len + max_new_token)."""
+    from moa_amd.attention.cache_utils import cache_config_summary, format_cache_summary
+    layers, model = cache_config_summary([[128, 1024, 128], [2624, 1152, 2560]], [[64] * 3] * 2, 5120)
+    assert layers[0]["cache_size"] == (pytest.approx(1280 / 3), 128, 1024)
+    assert layers[1]["circular_size"] == (pytest.approx(2048.0), 1088, 2560)
+    assert layers[0]["ratio"][2] == pytest.approx(0.2) and layers[0]["raw_cache_size"][0] == 5120
+    assert model["cache_size"] == (pytest.approx(7616 / 6), 128, 2624) and model["static_size"] == (64, 64, 64)
+    text = format_cache_summary(layers, model)
+    assert text.splitlines()[0].split()[:2] == ["layer_id", "raw_cache_size"] and "circular_size" in text
