@@ -46,19 +46,25 @@
 
 namespace moa {
 
-constexpr int kPfThreads = 512;
-constexpr int kQRows = 256;   // query rows per work-group
 constexpr int kWRows = 32;    // query rows per wave
 constexpr int kKV = 64;       // keys per tile (the sparsity block)
-constexpr int kStages = 4;    // LDS stages per tensor
+// Two shapes of work-group (NW waves, S LDS stages per tensor):
+//   8 waves, 4 stages: 256 query rows, one work-group per CU, the two halves of the work-group ping-pong
+//                      between matrix and softmax phase under one barrier per tile;
+//   4 waves, 2 stages: 128 query rows, two work-groups per CU (half the LDS and half the waves each), which
+//                      share the SIMDs the way the two halves do but are not tied to each other: while one
+//                      of them starts, ends or waits for the dispatcher the other has the CU to itself.
+#ifndef MOA_PF_WAVES
+#define MOA_PF_WAVES 8
+#endif
 constexpr int kMaxSortedHeads = 512;   // kv heads the span-sorted schedule handles (else: given order)
 
 struct Strides4 {
   int64_t b, h, n;
 };
 
-template <typename T, int D>
-__global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
+template <typename T, int D, int NW, int S>
+__global__ __launch_bounds__(NW * 64, 8 / NW) void prefill_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
     uint16_t* __restrict__ o, Strides4 qs, Strides4 ks, Strides4 vs, Strides4 os, int BH, int Hq,
     int group, int N, int n_qtiles, const int64_t* __restrict__ sink_blocks,
@@ -66,7 +72,13 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
   constexpr int KS = D / 16;          // MFMA k-steps of the QK^T product
   constexpr int DT = D / 32;          // 32-wide d tiles of the output
   constexpr int CPR = D / 8;          // 16-byte chunks per K/V row
-  constexpr int LPW = CPR / 8;        // async copies per wave per tile and tensor (64 chunks each)
+  constexpr int kPfThreads = NW * 64;
+  constexpr int kQRows = NW * kWRows; // query rows per work-group
+  constexpr int kQBlocks = kQRows / kKV;   // 64-row query blocks per work-group (two waves each)
+  constexpr int kStages = S;          // LDS stages per tensor
+  constexpr int LPW = CPR / NW;       // async copies per wave per tile and tensor (64 chunks each)
+  static_assert(NW == 4 || NW == 8, "4 or 8 waves");
+  static_assert(S == 2 || S == 4, "the stage ring is a power of two");
   constexpr int TILE_B = kKV * D * 2; // bytes of one K or V stage (rows unpadded)
   constexpr int ROW_B = D * 2;
   constexpr int RSH = 16 / CPR;       // rows per 256 bytes of LDS (1 at D=128, 2 at D=64)
@@ -130,15 +142,15 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
 
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int grp = wave >> 2;    // 0: group A, 1: group B (one phase behind A)
+  const int grp = wave >> 2;    // 0: group A, 1: group B (one phase behind A); four waves: all A
   const int mcol = lane & 31;   // query row inside the wave's 32 (the MFMA column)
   const int g = lane >> 5;      // half-wave
 
   const int ns = __builtin_amdgcn_readfirstlane(sorted ? s_ns[hk] : clamp_blocks(sink_blocks[hk]));
   const int nl = __builtin_amdgcn_readfirstlane(sorted ? s_nl[hk] : clamp_blocks(local_blocks[hk]));
-  const int mb0 = 4 * qt;                                  // first query block of the group
-  const int mbl = min(4 * qt + 3, nb - 1);                 // last one that exists
-  const int mbw = 4 * qt + (wave >> 1);                    // this wave's query block
+  const int mb0 = kQBlocks * qt;                           // first query block of the group
+  const int mbl = min(kQBlocks * qt + kQBlocks - 1, nb - 1);   // last one that exists
+  const int mbw = kQBlocks * qt + (wave >> 1);             // this wave's query block
   const bool wave_has_rows = mbw < nb;
 
   // tiles of the work-group: sinks [0, hi1], then band [lo2, mbl]
@@ -226,16 +238,19 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
   constexpr uint32_t kRing = kStages * TILE_B;                       // bytes of one tensor's ring (a power of two)
   const uint32_t k_dst0 = lds_address(s_k) + wave * LPW * 1024;      // this wave's share of stage 0
   const uint32_t v_dst0 = lds_address(s_v) + wave * LPW * 1024;
-  int j_0 = tile_at(0), j_1 = next_tile(j_0, 1), j_2 = next_tile(j_1, 2), j_3 = next_tile(j_2, 3);   // tiles of steps t .. t+3
+  int jt[S];   // tiles of steps t .. t+S-1
+  jt[0] = tile_at(0);
+#pragma unroll
+  for (int i = 1; i < S; ++i) jt[i] = next_tile(jt[i - 1], i);
 
-  // The matrix phase of iteration t reads K(t) and V(t-1) and starts the copies of K(t+3) and
-  // V(t+2), whose stages were last read in iteration t-1 by both groups.  Before the loop:
-  // K(0..2), V(0..1).
-  issue_tile(kbase, k_tile_bytes, ks.n, koff, true, j_0, k_dst0);
-  issue_tile(vbase, v_tile_bytes, vs.n, voff, false, j_0, v_dst0);
-  issue_tile(kbase, k_tile_bytes, ks.n, koff, true, j_1, k_dst0 + TILE_B);
-  issue_tile(vbase, v_tile_bytes, vs.n, voff, false, j_1, v_dst0 + TILE_B);
-  issue_tile(kbase, k_tile_bytes, ks.n, koff, true, j_2, k_dst0 + 2 * TILE_B);
+  // The matrix phase of iteration t reads K(t) and V(t-1) and starts the copies of K(t+S-1) and
+  // V(t+S-2), whose stages were last read in iteration t-1 by every wave.  Before the loop:
+  // K(0..S-2), V(0..S-3).
+#pragma unroll
+  for (int i = 0; i + 1 < S; ++i) {
+    issue_tile(kbase, k_tile_bytes, ks.n, koff, true, jt[i], k_dst0 + i * TILE_B);
+    if (i + 2 < S) issue_tile(vbase, v_tile_bytes, vs.n, voff, false, jt[i], v_dst0 + i * TILE_B);
+  }
 
   // ---- Q fragment (B operand): Q[m][16*ks + 8*g .. +7] ---------------------
   u32x4 qf[KS];
@@ -407,26 +422,26 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
   // barrier t-1; the copies started two iterations ago (K(t+1), V(t)) are first read after barrier
   // t, and every wave waits for its own before it.  Iteration n_tiles only finishes P.V of the
   // last tile.
-  uint32_t cst = 3 * TILE_B;   // ring offset of the stage K(t+3) is copied into; V(t+2) goes one stage below
+  uint32_t cst = (S - 1) * TILE_B;   // ring offset of the stage K(t+S-1) is copied into; V(t+S-2) goes one stage below
   uint32_t rst = 0;            // ring offset of the stage K(t) is read from
   int kd_prev = 0;             // how far the K read addresses moved in the previous iteration
   bool lc_prev = false;        // was tile t-1 live for this wave
   auto iteration = [&](int t, auto FIRST) __attribute__((always_inline)) {
     constexpr bool kFirst = decltype(FIRST)::value != 0;
-    constexpr int n_wait = 4 * LPW;   // the copies of this iteration and the one before may still be in flight
+    constexpr int n_wait = (S - 2) * 2 * LPW;   // copies started in the last S-2 iterations may still be in flight
     // ---------------- matrix phase ----------------
-    issue_tile(kbase, k_tile_bytes, ks.n, koff, true, j_3, k_dst0 + cst);
-    issue_tile(vbase, v_tile_bytes, vs.n, voff, false, j_2, v_dst0 + ((cst - TILE_B) & (kRing - 1)));
-    const bool lp = lc_prev, lc = (t < n_tiles) && live_tile(j_0);
+    issue_tile(kbase, k_tile_bytes, ks.n, koff, true, jt[S - 1], k_dst0 + cst);
+    issue_tile(vbase, v_tile_bytes, vs.n, voff, false, jt[S - 2], v_dst0 + ((cst - TILE_B) & (kRing - 1)));
+    const bool lp = lc_prev, lc = (t < n_tiles) && live_tile(jt[0]);
     if (kFirst) {
       if (lc) qk_phase();
     } else {
       if (lp || lc) matrix_phase();
     }
-    if (grp == 1) { wait_vm(n_wait); phase_barrier(); }
+    if (NW == 8 && grp == 1) { wait_vm(n_wait); phase_barrier(); }
     // ---------------- softmax phase ----------------
     if (lc) {
-      softmax(j_0);
+      softmax(jt[0]);
     } else if (lp) {   // the next matrix phase this wave runs must add nothing for a dead tile
 #pragma unroll
       for (int i = 0; i < 16; ++i) pf[i] = 0;
@@ -444,12 +459,11 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
       rst = (rst + TILE_B) & (kRing - 1);
       cst = (cst + TILE_B) & (kRing - 1);
       lc_prev = lc;
-      j_0 = j_1;
-      j_1 = j_2;
-      j_2 = j_3;
-      j_3 = next_tile(j_3, t + 4);
+#pragma unroll
+      for (int i = 0; i + 1 < S; ++i) jt[i] = jt[i + 1];
+      jt[S - 1] = next_tile(jt[S - 1], t + S);
     }
-    if (grp == 0) { wait_vm(n_wait); phase_barrier(); }
+    if (NW == 4 || grp == 0) { wait_vm(n_wait); phase_barrier(); }
   };
   iteration(0, IC<1>{});   // no P.V yet (and no V stage to read)
   for (int t = 1; t <= n_tiles; ++t) iteration(t, IC<0>{});
@@ -472,9 +486,9 @@ __global__ __launch_bounds__(kPfThreads, 1) void prefill_kernel(
     }
 }
 
-template <typename T, int D>
+template <int D, int S>
 static size_t prefill_lds_bytes() {
-  return (size_t)2 * kStages * kKV * D * sizeof(uint16_t);   // K stages + V stages
+  return (size_t)2 * S * kKV * D * sizeof(uint16_t);   // K stages + V stages
 }
 
 template <typename T, int D>
@@ -482,6 +496,8 @@ static int launch_prefill(const void* q, const void* k, const void* v, void* o, 
                           const int64_t* ks, const int64_t* vs, const int64_t* os, int B, int Hq,
                           int Hkv, int N, const int64_t* sink_blocks, const int64_t* local_blocks,
                           float sm_scale, hipStream_t st) {
+  constexpr int NW = MOA_PF_WAVES, S = NW / 2;
+  constexpr int kQRows = NW * kWRows;
   const int n_qtiles = (N + kQRows - 1) / kQRows;
   const int BH = B * Hq;
   const int64_t groups = (int64_t)((BH + 7) / 8) * 8 * n_qtiles;
@@ -491,11 +507,11 @@ static int launch_prefill(const void* q, const void* k, const void* v, void* o, 
     return fail(MOA_ERR_UNSUPPORTED, "moa_prefill_fwd: k/v token stride too large");
   Strides4 sq = {qs[0], qs[1], qs[2]}, sk = {ks[0], ks[1], ks[2]}, sv = {vs[0], vs[1], vs[2]},
            so = {os[0], os[1], os[2]};
-  const size_t lds = prefill_lds_bytes<T, D>();
+  const size_t lds = prefill_lds_bytes<D, S>();
   static bool lds_reserved[kMaxDevices] = {};   // per template instance
-  if (int rc = reserve_lds(reinterpret_cast<const void*>(&prefill_kernel<T, D>), lds, lds_reserved, "moa_prefill_fwd"))
+  if (int rc = reserve_lds(reinterpret_cast<const void*>(&prefill_kernel<T, D, NW, S>), lds, lds_reserved, "moa_prefill_fwd"))
     return rc;
-  hipLaunchKernelGGL((prefill_kernel<T, D>), dim3((unsigned)groups), dim3(kPfThreads), lds, st,
+  hipLaunchKernelGGL((prefill_kernel<T, D, NW, S>), dim3((unsigned)groups), dim3(NW * 64), lds, st,
                      (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (uint16_t*)o, sq, sk, sv,
                      so, BH, Hq, Hq / Hkv, N, n_qtiles, sink_blocks, local_blocks, mfma_softmax_scale(sm_scale));
   return check_launch("moa_prefill_fwd");
