@@ -82,7 +82,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void prefill_kernel(
   constexpr int TILE_B = kKV * D * 2; // bytes of one K or V stage (rows unpadded)
   constexpr int ROW_B = D * 2;
   constexpr int RSH = 16 / CPR;       // rows per 256 bytes of LDS (1 at D=128, 2 at D=64)
-  constexpr float kRescaleStep = 8.f; // rescale O only when a row max grew by more than 2^8
+  constexpr float kRescaleLimit = 256.f;   // the reference exponent is raised (and O rescaled) when a lane's 32 weights sum to more
   // The row maximum is taken over the unscaled scores, which needs a scale >= 0: a negative softmax
   // scale is moved into Q (sign bits of the packed 16-bit elements flipped, exact) and its magnitude kept.
   const float scale_log2 = __builtin_fabsf(scale_log2_signed);
@@ -274,7 +274,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void prefill_kernel(
   uint32_t pf[16];           // P^T of the current tile, packed pairs, B-operand order
 #pragma unroll
   for (int i = 0; i < 16; ++i) pf[i] = 0;
-  float m_run = -INFINITY;   // reference exponent of exp2: an integer >= the max of scale_log2 * s when set, then lagging it by <= kRescaleStep
+  float m_run = -INFINITY;   // reference exponent of exp2: an integer, ceil of the row max of scale_log2 * s when it was last set; a later max may pass it by < 8
   float l_run = 0.f;         // this lane's share of the running sum (the lane+32 twin holds the rest)
 
   // ---- operand read addresses: LDS byte address of stage 0, row 0 of this lane; stage, half and
@@ -368,17 +368,40 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void prefill_kernel(
         for (int i = 0; i < 16; ++i)
           if (nt * 32 + 8 * (i >> 2) + (i & 3) > thr) st[nt][i] = -INFINITY;
     }
-    float mx = st[0][0];
+    // Row sums are plain fp32 adds of the unrounded weights.  (v_dot2_f32_{f16,bf16} of the packed
+    // pair with a pair of ones would halve the instruction count, but those instructions stall the
+    // MFMA stream of the wave that shares the SIMD: measured 20 % slower per iteration.)
+    float psum[2];
+    auto weights = [&]() __attribute__((always_inline)) {
+      psum[0] = psum[1] = 0.f;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+      for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, st[nt][i]);
-    mx = max_with_other_half(mx);
-    const float m_cand = mx * scale_log2;   // finite: a live tile has a visible key in every row
-    if (__any(m_cand > m_run + kRescaleStep)) {
+        for (int i = 0; i < 16; i += 2) {
+          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i], scale_log2, -m_run));
+          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i + 1], scale_log2, -m_run));
+          pf[nt * 8 + (i >> 1)] = T::pack_rne(p0, p1);
+          psum[0] += p0;
+          psum[1] += p1;
+        }
+    };
+    // The common case needs no row maximum: weights are formed against the reference exponent as it
+    // stands, and their sum tells whether that was good enough.  A lane's 32 weights are >= 0, so a sum of
+    // at most 2^8 bounds each of them by 2^8 (the 16-bit types hold that with room to spare); a larger
+    // sum, or the first live tile (the reference is still -inf and the sum is inf or NaN; the file is
+    // compiled without NaN semantics, so that case is asked for by name), takes the path below.
+    weights();
+    if (__builtin_expect(__any(m_run == -INFINITY || psum[0] + psum[1] > kRescaleLimit), 0)) {
+      float mx = st[0][0];
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, st[nt][i]);
+      mx = max_with_other_half(mx);
+      const float m_cand = mx * scale_log2;   // finite: a live tile has a visible key in every row
       // The reference exponent stays an INTEGER: a weight is then 2^frac * 2^int, and its rounding to the
-      // storage type below does not depend on the power of two, so the rounded weights (relative to the
-      // row's sum) do not depend on the tile order or on how far m_run lags behind the true maximum.
+      // storage type does not depend on the power of two, so the rounded weights (relative to the row's
+      // sum) do not depend on the tile order or on how far m_run lags behind the true maximum.
       const float m_new = __builtin_ceilf(fmaxf(m_run, m_cand));
       const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
       l_run *= alpha;
@@ -387,21 +410,8 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void prefill_kernel(
 #pragma unroll
         for (int i = 0; i < 16; ++i) oacc[t][i] *= alpha;
       m_run = m_new;
+      weights();
     }
-    // Row sums are plain fp32 adds of the unrounded weights.  (v_dot2_f32_{f16,bf16} of the packed
-    // pair with a pair of ones would halve the instruction count, but those instructions stall the
-    // MFMA stream of the wave that shares the SIMD: measured 20 % slower per iteration.)
-    float psum[2] = {0.f, 0.f};
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int i = 0; i < 16; i += 2) {
-        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i], scale_log2, -m_run));
-        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[nt][i + 1], scale_log2, -m_run));
-        pf[nt * 8 + (i >> 1)] = T::pack_rne(p0, p1);
-        psum[0] += p0;
-        psum[1] += p1;
-      }
     l_run += psum[0] + psum[1];
   };
 
