@@ -453,8 +453,11 @@ __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
 #ifndef MOA_GQA_CHUNK
 #define MOA_GQA_CHUNK 2048
 #endif
+// Work-groups per CU the grid may hold.  A CU runs one at a time (the LDS rings fill it), so the hardware
+// dispatcher hands out chunks as CUs become free when every chunk is a work-group of its own: 602 us at
+// batch 64 of the 70B shape against 612-628 us with 2-16 per CU, each walking several chunks in a fixed order.
 #ifndef MOA_GQA_BLOCKS
-#define MOA_GQA_BLOCKS 4
+#define MOA_GQA_BLOCKS 64
 #endif
 // Cache rows per work-group step (a quarter per wave).  A chunk start costs a wave full memory
 // latencies with nothing in flight, so long chunks win: 2048 is the best of 512..4096 at batch 64 and at
@@ -467,14 +470,20 @@ constexpr int kGqaMaxG = 8;       // query heads per ring the per-wave result bu
 #endif
 constexpr int kGqaWaves = MOA_GQA_WAVES;          // waves per work-group
 constexpr int kGqaThreads = 64 * kGqaWaves;
-constexpr int kGqaStages = 8 / kGqaWaves;         // LDS stages per wave (8 stages of 16 KiB at D = 128 in all)
+#ifndef MOA_GQA_STAGES
+#define MOA_GQA_STAGES (8 / MOA_GQA_WAVES)
+#endif
+#ifndef MOA_GQA_LDS_STAGES
+#define MOA_GQA_LDS_STAGES MOA_GQA_STAGES
+#endif
+constexpr int kGqaStages = MOA_GQA_STAGES;        // LDS stages per wave (8 stages of 16 KiB at D = 128 in all)
 
 template <typename T> struct MfmaElem;
 template <> struct MfmaElem<F16> { typedef PF16 type; };
 template <> struct MfmaElem<BF16> { typedef PBF16 type; };
 
 template <int D>
-constexpr size_t gqa_lds_bytes() { return (size_t)kGqaWaves * kGqaStages * 2 * kGqaTile * D * 2; }
+constexpr size_t gqa_lds_bytes() { return (size_t)kGqaWaves * MOA_GQA_LDS_STAGES * 2 * kGqaTile * D * 2; }
 
 template <typename T, int D, int CHUNK>
 __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
@@ -783,7 +792,7 @@ static int launch_decode_gqa_chunk(const void* q, const void* kc, const void* vc
                                    int H, int G, int64_t sumC, float sm_scale, hipStream_t st) {
   const int cap = (int)decode_cap(sumC, H);   // partial slots per batch row the workspace was sized for
   const int64_t chunks = (sumC + CHUNK - 1) / CHUNK + H;   // at most this many steps per batch row
-  int bx = (int)((256 * MOA_GQA_BLOCKS + B - 1) / B);   // one work-group per CU at a time (its LDS ring fills the CU)
+  int bx = (int)((256 * MOA_GQA_BLOCKS + B - 1) / B);   // in practice one work-group per chunk (see MOA_GQA_BLOCKS)
   if (bx > chunks) bx = (int)chunks;
   if (bx < 1) bx = 1;
   constexpr size_t lds = gqa_lds_bytes<D>();
