@@ -105,6 +105,31 @@ def test_random_plans_against_oracle(dev, seed):
     check_prefill(out, q, k, v, sm, ns, nl, (seed, N, D, ns, nl))
 
 
+@pytest.mark.parametrize("layout", ["fused_qkv", "contiguous_bhnd"])
+def test_operand_layouts(dev, layout):
+    """q, k, v as the three column slices of ONE fused projection output [B, N, (Hq + 2 Hkv) D] (token
+    stride is that of the fused row, the slices start at different 16-byte-aligned offsets), and as
+    contiguous [B, H, N, D] tensors (what a caller gets after .contiguous()): the operator takes both
+    through their strides, without a copy."""
+    B, Hq, Hkv, N, D = 2, 8, 2, 333, 128
+    dtype = torch.float16
+    g = torch.Generator().manual_seed(11)
+    if layout == "fused_qkv":
+        fused = torch.randn(B, N, (Hq + 2 * Hkv) * D, generator=g).to(dev, dtype)
+        q = fused[..., :Hq * D].view(B, N, Hq, D).transpose(1, 2)
+        k = fused[..., Hq * D:(Hq + Hkv) * D].view(B, N, Hkv, D).transpose(1, 2)
+        v = fused[..., (Hq + Hkv) * D:].view(B, N, Hkv, D).transpose(1, 2)
+        assert q.stride(2) == (Hq + 2 * Hkv) * D and not k.is_contiguous()
+    else:
+        q = torch.randn(B, Hq, N, D, generator=g).to(dev, dtype)
+        k = torch.randn(B, Hkv, N, D, generator=g).to(dev, dtype)
+        v = torch.randn(B, Hkv, N, D, generator=g).to(dev, dtype)
+    ns, nl = [1, 0], [2, 4]
+    sm = D ** -0.5
+    out = _run(q, k, v, sm, ns, nl, dev)
+    check_prefill(out, q, k, v, sm, ns, nl, ("layout", layout))
+
+
 def test_dead_rows_are_zero(dev):
     """ns = nl = 0 sees nothing; nl = 0 with sinks sees only sink blocks."""
     q, k, v = _qkv(1, 2, 256, 128, torch.float16, dev, seed=3)
