@@ -2,6 +2,7 @@
 
     python -m moa_amd.build            # build if sources are newer than the library
     python -m moa_amd.build --force    # always rebuild
+    python -m moa_amd.build --experiment -DNAME ...   # rebuild with extra hipcc flags (measurements only)
 
 hipcc cross-compiles without a GPU.  The library is kept in-tree next to this
 file so that it travels with the source tree.
@@ -12,6 +13,7 @@ import os
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
+from typing import Sequence
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
@@ -56,9 +58,8 @@ def is_stale() -> bool:
     return (not os.path.exists(LIB_PATH)) or os.path.getmtime(LIB_PATH) < _deps_mtime()
 
 
-def _compile(src: str) -> str:
+def _compile(src: str, extra: Sequence[str] = ()) -> str:
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    extra = os.environ.get("MOA_HIPCC_FLAGS", "").split()   # e.g. -DNAME for an experiment build
     cmd = [_hipcc(), *HIPCC_FLAGS, *PER_SOURCE_FLAGS.get(src, []), *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -70,8 +71,10 @@ def _compile(src: str) -> str:
     return obj
 
 
-def build(force: bool = False, verbose: bool = True) -> str:
-    if not force and not is_stale():
+def build(force: bool = False, verbose: bool = True, experiment_flags: Sequence[str] = ()) -> str:
+    """Compiles every source and links the library.  ``experiment_flags`` (extra hipcc arguments) are for
+    measurement builds only and must be asked for explicitly: the environment never changes the build."""
+    if not force and not experiment_flags and not is_stale():
         return LIB_PATH
     os.makedirs(OBJ_DIR, exist_ok=True)
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
@@ -79,7 +82,7 @@ def build(force: bool = False, verbose: bool = True) -> str:
     if missing:
         raise RuntimeError(f"missing sources: {sorted(missing)}")
     with ThreadPoolExecutor(max_workers=min(4, len(srcs))) as ex:
-        objs = list(ex.map(_compile, srcs))
+        objs = list(ex.map(lambda s: _compile(s, experiment_flags), srcs))
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -90,4 +93,6 @@ def build(force: bool = False, verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
-    build(force="--force" in sys.argv)
+    argv = sys.argv[1:]
+    flags = argv[argv.index("--experiment") + 1:] if "--experiment" in argv else []
+    build(force="--force" in argv or bool(flags), experiment_flags=flags)

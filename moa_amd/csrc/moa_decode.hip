@@ -40,10 +40,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kDecThreads = 256;
 constexpr int kDecWaves = kDecThreads / 64;
-#ifndef MOA_DEC_BATCH
-#define MOA_DEC_BATCH 8
-#endif
-constexpr int kBatch = MOA_DEC_BATCH;   // wave-wide loads in flight per tensor
+constexpr int kBatch = 8;           // wave-wide loads in flight per tensor
 constexpr int kMaxHeads = 256;     // heads per batch row the LDS prefix covers
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -450,40 +447,26 @@ __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
 // private two-stage LDS ring with asynchronous copies (16-byte chunks XOR-permuted as in the
 // prefill kernel), so no work-group barrier is needed inside the loop.  Chunks, partials and the
 // merge kernel are those of the vector version, with a longer chunk.
-#ifndef MOA_GQA_CHUNK
-#define MOA_GQA_CHUNK 2048
-#endif
 // Work-groups per CU the grid may hold.  A CU runs one at a time (the LDS rings fill it), so the hardware
 // dispatcher hands out chunks as CUs become free when every chunk is a work-group of its own: 602 us at
 // batch 64 of the 70B shape against 612-628 us with 2-16 per CU, each walking several chunks in a fixed order.
-#ifndef MOA_GQA_BLOCKS
-#define MOA_GQA_BLOCKS 64
-#endif
+constexpr int kGqaBlocksPerCu = 64;
 // Cache rows per work-group step (a quarter per wave).  A chunk start costs a wave full memory
 // latencies with nothing in flight, so long chunks win: 2048 is the best of 512..4096 at batch 64 and at
 // batch 4.
-constexpr int kGqaChunk = MOA_GQA_CHUNK;
+constexpr int kGqaChunk = 2048;
 constexpr int kGqaTile = 32;      // keys per MFMA tile
 constexpr int kGqaMaxG = 8;       // query heads per ring the per-wave result buffers are sized for
-#ifndef MOA_GQA_WAVES
-#define MOA_GQA_WAVES 4
-#endif
-constexpr int kGqaWaves = MOA_GQA_WAVES;          // waves per work-group
+constexpr int kGqaWaves = 4;      // waves per work-group (8 waves with one stage each measure the same)
 constexpr int kGqaThreads = 64 * kGqaWaves;
-#ifndef MOA_GQA_STAGES
-#define MOA_GQA_STAGES (8 / MOA_GQA_WAVES)
-#endif
-#ifndef MOA_GQA_LDS_STAGES
-#define MOA_GQA_LDS_STAGES MOA_GQA_STAGES
-#endif
-constexpr int kGqaStages = MOA_GQA_STAGES;        // LDS stages per wave (8 stages of 16 KiB at D = 128 in all)
+constexpr int kGqaStages = 2;     // LDS stages per wave (8 stages of 16 KiB at D = 128 in all)
 
 template <typename T> struct MfmaElem;
 template <> struct MfmaElem<F16> { typedef PF16 type; };
 template <> struct MfmaElem<BF16> { typedef PBF16 type; };
 
 template <int D>
-constexpr size_t gqa_lds_bytes() { return (size_t)kGqaWaves * MOA_GQA_LDS_STAGES * 2 * kGqaTile * D * 2; }
+constexpr size_t gqa_lds_bytes() { return (size_t)kGqaWaves * kGqaStages * 2 * kGqaTile * D * 2; }
 
 template <typename T, int D, int CHUNK>
 __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
@@ -720,19 +703,10 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
   }
 }
 
-#ifndef MOA_DEC_CHUNK
-#define MOA_DEC_CHUNK 512
-#endif
-#ifndef MOA_DEC_BLOCKS
-#define MOA_DEC_BLOCKS 16
-#endif
-#ifndef MOA_DEC_SMALL_BELOW
-#define MOA_DEC_SMALL_BELOW 2   // work-groups per CU below which the chunks are half as long
-#endif
-#ifndef MOA_DEC_PIPE_FROM
-#define MOA_DEC_PIPE_FROM 3   // work-groups per CU from which the waves pipeline their own loads
-#endif
-constexpr int kChunk = MOA_DEC_CHUNK;
+constexpr int kChunk = 512;           // cache rows per work-group step of the one-query-head kernel
+constexpr int kDecBlocksPerCu = 16;   // work-groups per CU over the whole grid
+constexpr int kDecSmallBelow = 2;     // work-groups per CU below which the chunks are half as long
+constexpr int kDecPipeFrom = 3;       // work-groups per CU from which the waves pipeline their own loads
 
 constexpr int kSmallChunk = kChunk / 2;   // chunk length of the one-query-head kernel when the grid is small
 
@@ -752,12 +726,12 @@ static int launch_decode(const void* q, const void* kc, const void* vc, void* o,
   const int64_t chunks = (sumC + kChunk - 1) / kChunk + H;   // per batch row, at the normal chunk length
   // 16 work-groups per CU over the whole grid (measured: 8 leaves a visible tail, 32 is no better),
   // never more per batch row than chunks exist
-  int bx = (int)((256 * MOA_DEC_BLOCKS + B - 1) / B);
+  int bx = (int)((256 * kDecBlocksPerCu + B - 1) / B);
   if (bx > cap) bx = cap;
   if (bx < 1) bx = 1;
-  const bool pipe = (int64_t)B * chunks >= (int64_t)256 * MOA_DEC_PIPE_FROM;
+  const bool pipe = (int64_t)B * chunks >= (int64_t)256 * kDecPipeFrom;
   // fewer than two work-groups per CU: half-length chunks give every CU something to do
-  const bool small = (int64_t)B * chunks < (int64_t)256 * MOA_DEC_SMALL_BELOW;
+  const bool small = (int64_t)B * chunks < (int64_t)256 * kDecSmallBelow;
   constexpr int GROUPS = kDecThreads / D;
   const int mx = (H * G + GROUPS - 1) / GROUPS;
   if (small) {
@@ -792,7 +766,7 @@ static int launch_decode_gqa_chunk(const void* q, const void* kc, const void* vc
                                    int H, int G, int64_t sumC, float sm_scale, hipStream_t st) {
   const int cap = (int)decode_cap(sumC, H);   // partial slots per batch row the workspace was sized for
   const int64_t chunks = (sumC + CHUNK - 1) / CHUNK + H;   // at most this many steps per batch row
-  int bx = (int)((256 * MOA_GQA_BLOCKS + B - 1) / B);   // in practice one work-group per chunk (see MOA_GQA_BLOCKS)
+  int bx = (int)((256 * kGqaBlocksPerCu + B - 1) / B);   // in practice one work-group per chunk (see kGqaBlocksPerCu)
   if (bx > chunks) bx = (int)chunks;
   if (bx < 1) bx = 1;
   constexpr size_t lds = gqa_lds_bytes<D>();
@@ -819,13 +793,8 @@ static int launch_decode_gqa(const void* q, const void* kc, const void* vc, void
   // 2048-row chunk per CU): 49.8 us per call with 2048-row chunks, 53.3 with 1024, 62.3 with 512 -- a chunk
   // start costs three dependent memory latencies (ring index, query rows, first tiles), which shorter
   // chunks pay more often than they win in balance.
-#define MOA_GQA_CALL(CH) \
-  launch_decode_gqa_chunk<T, D, CH>(q, kc, vc, o, part_acc, part_ml, head_start, head_valid, B, H, G, sumC, sm_scale, st)
-#ifdef MOA_GQA_FORCE_CHUNK   // experiment builds
-  return MOA_GQA_CALL(MOA_GQA_FORCE_CHUNK);
-#endif
-  return MOA_GQA_CALL(kGqaChunk);
-#undef MOA_GQA_CALL
+  return launch_decode_gqa_chunk<T, D, kGqaChunk>(q, kc, vc, o, part_acc, part_ml, head_start, head_valid, B, H, G, sumC,
+                                                  sm_scale, st);
 }
 
 // Launches the decode kernels with their partials in `workspace` (at least

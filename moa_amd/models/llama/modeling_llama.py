@@ -124,11 +124,12 @@ def install_plan(attention_layers: List[nn.Module], moa_config: Dict, permute_he
 
 
 def new_cache_for_plan(moa_config: Dict, max_new_token: int, batch_size: int, seq_len: int, head_dim: int,
-                       device, dtype) -> StaticCircularCache:
+                       device, dtype, verbose: bool = False) -> StaticCircularCache:
     """The cache the reference's model forward builds at the start of a generation
-    (modeling_llama.py:93-112): sizes from the plan at this prompt length."""
+    (modeling_llama.py:93-112): sizes from the plan at this prompt length.  ``verbose`` prints the
+    cache-size summary, as the reference does when ``moa_verbose`` was set (:95-104)."""
     cfg = moa_config_to_cache_config(moa_config, seq_len, max_new_token=max_new_token, sink_size=64,
-                                     minimum_cache_size=128, split_size=64, verbose=False)
+                                     minimum_cache_size=128, split_size=64, verbose=verbose)
     return StaticCircularCache(cache_size=cfg["cache_size"], static_size=cfg["static_size"], batch_size=batch_size,
                                head_dim=head_dim, device=device, dtype=dtype)
 
@@ -323,14 +324,29 @@ def _rope_base(config) -> float:
 
 
 def LlamaModel_MixtureAttention_forward(self, input_ids=None, attention_mask=None, position_ids=None,
-                                        past_key_values=None, inputs_embeds=None, use_cache=None, **kwargs):
+                                        past_key_values=None, inputs_embeds=None, use_cache=None,
+                                        output_attentions=None, output_hidden_states=None, return_dict=None,
+                                        cache_position=None, **kwargs):
     """Model forward with the MoA attention path (reference modeling_llama.py:52-204): builds the
     StaticCircularCache from the plan at the first call of a generation (any other kind of cache passed
-    in is replaced, as in the reference :93-112), continues the positions from the cache, runs the
-    decoder layers with the attention of ``mixture_attention_forward``.  Returns an object with
-    ``last_hidden_state`` (only the last position when ``last_hidden_only`` was set, :188-190) and
-    ``past_key_values`` (the StaticCircularCache)."""
+    in -- ``generate`` of transformers hands over its own empty one -- is replaced, as in the reference
+    :93-112; the cache summary is printed when ``moa_verbose`` was set), continues the positions from the
+    cache unless ``cache_position`` / ``position_ids`` say otherwise (:114-120), runs the decoder layers
+    with the attention of ``mixture_attention_forward``.  Returns a ``BaseModelOutputWithPast`` with
+    ``last_hidden_state`` (only the last position when ``last_hidden_only`` was set, :188-190),
+    ``past_key_values`` (the StaticCircularCache) and, when asked for, ``hidden_states``; a tuple of the
+    non-empty ones with ``return_dict=False`` (:183-184).  ``output_attentions`` raises, as in the
+    reference (:126-129)."""
     assert self.use_moa, "call set_mixture_of_attention first"
+    config = getattr(self, "config", None)
+    if output_attentions is None:
+        output_attentions = getattr(config, "output_attentions", False)
+    if output_hidden_states is None:
+        output_hidden_states = getattr(config, "output_hidden_states", False)
+    if return_dict is None:
+        return_dict = getattr(config, "use_return_dict", True)
+    if output_attentions:
+        raise NotImplementedError("output_attentions is not supported in mixture of attention")
     if (input_ids is None) == (inputs_embeds is None):
         raise ValueError("You must specify exactly one of input_ids or inputs_embeds")
     hidden_states = self.embed_tokens(input_ids) if inputs_embeds is None else inputs_embeds
@@ -338,29 +354,42 @@ def LlamaModel_MixtureAttention_forward(self, input_ids=None, attention_mask=Non
     _, _, head_dim = attention_geometry(self.layers[0].self_attn)
     if not isinstance(past_key_values, StaticCircularCache):
         past_key_values = new_cache_for_plan(self.moa_config, self.moa_max_new_token, bsz, q_len, head_dim,
-                                             hidden_states.device, hidden_states.dtype)
+                                             hidden_states.device, hidden_states.dtype,
+                                             verbose=getattr(self, "moa_verbose", False))
     if position_ids is None:
-        past = past_key_values.get_seq_length()
-        position_ids = torch.arange(past, past + q_len, device=hidden_states.device)[None, :]
-    if attention_mask is not None and not (attention_mask == 0).any():
-        attention_mask = None    # a mask without padding is no mask (:119-121)
+        if cache_position is None:
+            past = past_key_values.get_seq_length()
+            cache_position = torch.arange(past, past + q_len, device=hidden_states.device)
+        position_ids = cache_position[None, :]
+    # A mask without padding is no mask (:119-121).  A decode step needs none at all (the cache's decode
+    # branch ignores it, cache_utils.py:1020-1058), so only a prompt pays for looking at it.
+    if q_len == 1 or (attention_mask is not None and not (attention_mask == 0).any()):
+        attention_mask = None
     cos_sin = rotary_cos_sin(position_ids, head_dim, hidden_states.dtype, _rope_base(self.config))
+    all_hidden_states = () if output_hidden_states else None
     with torch.no_grad():
         for layer in self.layers:
+            if output_hidden_states:
+                all_hidden_states += (hidden_states,)
             residual = hidden_states
             hidden_states = residual + mixture_attention_forward(layer.self_attn, layer.input_layernorm(hidden_states),
                                                                  cos_sin, past_key_values, attention_mask)
             hidden_states = hidden_states + layer.mlp(layer.post_attention_layernorm(hidden_states))
         hidden_states = self.norm(hidden_states)
-    if self.last_hidden_only:
+    if output_hidden_states:
+        all_hidden_states += (hidden_states,)
+    if not return_dict:
+        return tuple(v for v in (hidden_states, past_key_values, all_hidden_states) if v is not None)
+    if getattr(self, "last_hidden_only", False):
         hidden_states = hidden_states[:, -1:, :]
     try:
         from transformers.modeling_outputs import BaseModelOutputWithPast
-        return BaseModelOutputWithPast(last_hidden_state=hidden_states, past_key_values=past_key_values)
+        return BaseModelOutputWithPast(last_hidden_state=hidden_states, past_key_values=past_key_values,
+                                       hidden_states=all_hidden_states)
     except ImportError:   # a duck-typed model without transformers installed
         from types import SimpleNamespace
         return SimpleNamespace(last_hidden_state=hidden_states, past_key_values=past_key_values,
-                               hidden_states=None, attentions=None)
+                               hidden_states=all_hidden_states, attentions=None)
 
 
 def LlamaModel_set_mixture_of_attention(self, moa_config: Dict, permute_head: bool = False, moa_verbose: bool = False,
