@@ -75,6 +75,13 @@ __device__ __forceinline__ void wait_vm(int n) {
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// The same for a count known at compile time.
+template <int N>
+__device__ __forceinline__ void wait_vm_exact() {
+  static_assert(N >= 0 && N < 64, "vmcnt holds 6 bits");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
 // Work-group barrier WITHOUT the memory fence of __syncthreads(): the fence would make every wave
 // wait for all of its outstanding async copies (vmcnt(0)) at each phase boundary and serialise the
 // copy pipeline.  What must be visible at a barrier is waited for explicitly with wait_vm().
@@ -102,6 +109,10 @@ struct IC {
 __device__ __forceinline__ u32x4 lds_load16(uint32_t addr, int imm) {
   typedef u32x4 __attribute__((address_space(3))) * lds_u32x4_ptr;
   return *(lds_u32x4_ptr)(uintptr_t)(addr + imm);
+}
+__device__ __forceinline__ void lds_store8(uint32_t addr, u32x2 v) {
+  typedef u32x2 __attribute__((address_space(3))) * lds_u32x2_ptr;
+  *(lds_u32x2_ptr)(uintptr_t)addr = v;
 }
 // The transposing read: 4 consecutive rows of one 16-bit column out of a row-major LDS tile.  Within
 // each group of 16 lanes, lane i must point at (row0 + i/4, col0 + 4*(i%4)); it receives rows
