@@ -89,6 +89,9 @@ class StaticCircularCache:
 
         self.cache_position = 0
         self._kv_len = [0 for _ in range(self.num_layers)]
+        self._ready_on: List[Optional[torch.device]] = [None] * self.num_layers   # device the layer's tensors are on
+        self._step_args: List[Optional[Dict[str, Any]]] = [None] * self.num_layers   # what rope_update keeps per layer
+        self._capturing: Optional[bool] = None   # is the stream capturing (asked once per step)
 
         # K/V are created on the device of the first update of each layer
         self.key_cache: List[Optional[Tensor]] = [None] * self.num_layers
@@ -144,6 +147,8 @@ class StaticCircularCache:
 
     # ------------------------------------------------------------------
     def _to_device(self, layer_idx: int, device: torch.device) -> None:
+        if self._ready_on[layer_idx] == device:
+            return
         for name in ("mask_cache", "cache_update_index", "cache_head_start_index",
                      "circular_cache_head_index", "cache_valid_length", "cache_max_length",
                      "circular_cache_size", "static_cache_size", "head_index"):
@@ -154,6 +159,8 @@ class StaticCircularCache:
             shape = (self.batch_size, self.layer_cache_size[layer_idx], self.head_dim)
             self.key_cache[layer_idx] = torch.zeros(shape, dtype=self.dtype, device=device)
             self.value_cache[layer_idx] = torch.zeros(shape, dtype=self.dtype, device=device)
+        self._ready_on[layer_idx] = device
+        self._step_args[layer_idx] = None
 
     def _check_capture(self, layer_idx: int, device) -> None:
         """A decode step recorded into a HIP graph bakes in the host value ``kv_len``, which the
@@ -162,8 +169,12 @@ class StaticCircularCache:
         decision does not change any more, i.e. once every head of the layer is past its sinks.
         Capturing earlier would let replays walk a head's pointer linearly out of its segment.
         (Replays do not advance ``get_seq_length()`` / ``cache_position`` either: callers that replay
-        pass explicit positions.)"""
-        if torch.cuda.is_current_stream_capturing() and self._kv_len[layer_idx] + 1 <= self._max_static_size[layer_idx]:
+        pass explicit positions.)  Called before anything is changed, so a caller that catches the error
+        can go on eagerly.  The stream is asked once per step (layer 0); the other layers of the step
+        use that answer."""
+        if layer_idx == 0 or self._capturing is None:
+            self._capturing = torch.cuda.is_current_stream_capturing()
+        if self._capturing and self._kv_len[layer_idx] + 1 <= self._max_static_size[layer_idx]:
             raise RuntimeError(
                 f"StaticCircularCache: layer {layer_idx} has seen {self._kv_len[layer_idx]} tokens, not more than its "
                 f"largest static size {self._max_static_size[layer_idx]}: a decode step captured now would be "
@@ -187,7 +198,8 @@ class StaticCircularCache:
         where keys/values are what ``update`` returns.  With ``seq_len == 1`` this is ONE launch:
         q is rotated into a ``[batch, 1, q_heads, head_dim]`` buffer (returned as its
         ``[batch, q_heads, 1, head_dim]`` view, the layout the decode kernel takes without a copy), k is
-        rotated straight into its ring slot, v is copied into its slot.
+        rotated straight into its ring slot, v is copied into its slot.  That buffer belongs to the
+        cache, one per layer, and is written again by the layer's next step.
         """
         from ..kernels.rotary import apply_rotary_pos_emb, _cos_sin_strides
 
@@ -200,7 +212,7 @@ class StaticCircularCache:
         assert layer_idx < self.num_layers
         H = self.num_head_for_each_layer[layer_idx]
         device = key_states.device
-        if torch.device(device).type != "cuda":
+        if device.type != "cuda":
             raise _lib.MoaKernelError(
                 "StaticCircularCache.rope_update: tensors must live on the GPU; moa_amd has no CPU path")
         B, Hq, _, D = query_states.shape
@@ -208,32 +220,68 @@ class StaticCircularCache:
         assert B == self.batch_size and D == self.head_dim
         assert query_states.dtype == self.dtype and key_states.dtype == self.dtype and value_states.dtype == self.dtype
         assert cos.dtype == self.dtype and sin.dtype == self.dtype, "cos/sin must have the cache dtype"
-        lib = _lib.load()
         self._to_device(layer_idx, device)
+        self._check_capture(layer_idx, device)
+
+        # What does not change from step to step is kept per layer: the library handle, the pointers of the
+        # cache and its index tensors, the q buffer, and the stride arrays of the last operand layout seen.
+        st = self._step_args[layer_idx]
+        layout = (query_states.stride(), key_states.stride(), value_states.stride(), cos.shape, cos.stride(),
+                  sin.stride(), Hq)
+        if st is None or st["layout"] != layout:
+            qs, ks_, vs_ = query_states.stride(), key_states.stride(), value_states.stride()
+            if qs[-1] != 1 or ks_[-1] != 1 or vs_[-1] != 1:
+                st = None   # rare: operands without a contiguous head_dim are copied, nothing is kept
+            else:
+                upd = self.cache_update_index[layer_idx]
+                assert upd.is_contiguous() and self.cache_valid_length[layer_idx].is_contiguous()
+                _, _, css = _cos_sin_strides(cos, sin, B, 1, D)
+                q_out = torch.empty((B, 1, Hq, D), dtype=self.dtype, device=device)
+                st = {
+                    "layout": layout, "lib": _lib.load(), "q_out": q_out, "q_view": q_out.transpose(1, 2),
+                    "cos_ok": cos.stride(-1) == 1 and sin.stride() == cos.stride(),
+                    "strides": (_lib.i64_array((qs[0], qs[1], qs[3])), _lib.i64_array((ks_[0], ks_[1], ks_[3])),
+                                _lib.i64_array((vs_[0], vs_[1], vs_[3])), css[0]),
+                    "tail": (q_out.data_ptr(), self.key_cache[layer_idx].data_ptr(),
+                             self.value_cache[layer_idx].data_ptr(), self.mask_cache[layer_idx].data_ptr(),
+                             upd.data_ptr(), self.cache_valid_length[layer_idx].data_ptr(),
+                             self.circular_cache_head_index[layer_idx].data_ptr(),
+                             self.circular_cache_size[layer_idx].data_ptr(),
+                             self.static_cache_size[layer_idx].data_ptr(),
+                             self.cache_max_length[layer_idx].data_ptr()),
+                    "sizes": (B, Hq, H, D, self.layer_cache_size[layer_idx], _lib.dtype_code(self.dtype)),
+                }
+                self._step_args[layer_idx] = st
+        if st is not None and st["cos_ok"]:
+            qstr, kstr, vstr, cos_b = st["strides"]
+            rc = st["lib"].moa_rope_cache_append(
+                query_states.data_ptr(), key_states.data_ptr(), value_states.data_ptr(), qstr, kstr, vstr,
+                cos.data_ptr(), sin.data_ptr(), cos_b, *st["tail"], self._kv_len[layer_idx], *st["sizes"],
+                _lib.current_stream_ptr(device))
+            q_view = st["q_view"]
+        else:
+            cos, sin, css = _cos_sin_strides(cos, sin, B, 1, D)
+            qn, kn, vn = (t[:, :, -1, :] for t in (query_states, key_states, value_states))
+            qn, kn, vn = (t if t.stride(-1) == 1 else t.contiguous() for t in (qn, kn, vn))
+            q_out = torch.empty((B, 1, Hq, D), dtype=self.dtype, device=device)
+            rc = _lib.load().moa_rope_cache_append(
+                qn.data_ptr(), kn.data_ptr(), vn.data_ptr(), _lib.i64_array(qn.stride()), _lib.i64_array(kn.stride()),
+                _lib.i64_array(vn.stride()), cos.data_ptr(), sin.data_ptr(), css[0], q_out.data_ptr(),
+                self.key_cache[layer_idx].data_ptr(), self.value_cache[layer_idx].data_ptr(),
+                self.mask_cache[layer_idx].data_ptr(), self.cache_update_index[layer_idx].data_ptr(),
+                self.cache_valid_length[layer_idx].data_ptr(),
+                self.circular_cache_head_index[layer_idx].data_ptr(),
+                self.circular_cache_size[layer_idx].data_ptr(),
+                self.static_cache_size[layer_idx].data_ptr(),
+                self.cache_max_length[layer_idx].data_ptr(),
+                self._kv_len[layer_idx], B, Hq, H, D, self.layer_cache_size[layer_idx],
+                _lib.dtype_code(self.dtype), _lib.current_stream_ptr(device))
+            q_view = q_out.transpose(1, 2)
+        _lib.check(rc)
         if layer_idx == 0:
             self.cache_position += 1
-        self._check_capture(layer_idx, device)
-        cos, sin, css = _cos_sin_strides(cos, sin, B, 1, D)
-        qn, kn, vn = (t[:, :, -1, :] for t in (query_states, key_states, value_states))
-        qn, kn, vn = (t if t.stride(-1) == 1 else t.contiguous() for t in (qn, kn, vn))
-        q_out = torch.empty((B, 1, Hq, D), dtype=self.dtype, device=device)
-        upd = self.cache_update_index[layer_idx]
-        assert upd.is_contiguous() and self.cache_valid_length[layer_idx].is_contiguous()
-        rc = lib.moa_rope_cache_append(
-            qn.data_ptr(), kn.data_ptr(), vn.data_ptr(), _lib.i64_array(qn.stride()), _lib.i64_array(kn.stride()),
-            _lib.i64_array(vn.stride()), cos.data_ptr(), sin.data_ptr(), css[0], q_out.data_ptr(),
-            self.key_cache[layer_idx].data_ptr(), self.value_cache[layer_idx].data_ptr(),
-            self.mask_cache[layer_idx].data_ptr(), upd.data_ptr(),
-            self.cache_valid_length[layer_idx].data_ptr(),
-            self.circular_cache_head_index[layer_idx].data_ptr(),
-            self.circular_cache_size[layer_idx].data_ptr(),
-            self.static_cache_size[layer_idx].data_ptr(),
-            self.cache_max_length[layer_idx].data_ptr(),
-            self._kv_len[layer_idx], B, Hq, H, D, self.layer_cache_size[layer_idx],
-            _lib.dtype_code(self.dtype), _lib.current_stream_ptr(device))
-        _lib.check(rc)
         self._kv_len[layer_idx] += 1
-        return q_out.transpose(1, 2), self.key_cache[layer_idx], self.value_cache[layer_idx]
+        return q_view, self.key_cache[layer_idx], self.value_cache[layer_idx]
 
     def update(
         self,
@@ -278,6 +326,8 @@ class StaticCircularCache:
             batch_size = self.batch_size
             seq_len = key_states.shape[-2] if key_states is not None else 1
             head_dim = self.head_dim
+        if seq_len == 1:
+            self._check_capture(layer_idx, device)   # before anything is changed
         if layer_idx == 0:
             self.cache_position += seq_len
 
@@ -290,7 +340,6 @@ class StaticCircularCache:
         assert upd.is_contiguous() and self.cache_valid_length[layer_idx].is_contiguous()
 
         if seq_len == 1:
-            self._check_capture(layer_idx, device)
             kn = vn = None
             kns = vns = None
             if self.update_cache_content:

@@ -14,7 +14,14 @@ So there are two comparisons:
       the rounded weights independent of the order the keys are met in): the stated bound, every element;
   (2) against the exact oracle: every element inside the a-priori bound of the weight rounding plus
       the output rounding, 2^-8 * (attention of |V| + |ref|) + 2e-3; the elements outside the STATED
-      bound are counted and recorded, and at the benchmark's size their fraction is asserted.
+      bound are counted, recorded, and held to a rate in EVERY comparison: at most MAX_FRACTION of the
+      elements (with three standard deviations of counting noise on top, so that a comparison of a few
+      thousand elements is not failed by one element), 1e-5 at the benchmark's size where the callers say so.
+      Measured on the MI355X: 1.2e-4 at worst over the random plans (N = 65), 2.0e-4 with peaked scores,
+      6e-7 at the benchmark's size.  Normalising a row by the sum of the ROUNDED weights instead of the
+      exact sum does not change these counts (3 against 3, 25 against 24, 267 against 261 elements in a CPU
+      experiment over N = 65 .. 1024): the elements outside belong to rows in which two to six keys carry
+      the weight and their values cancel, and there the relative error 2^-9 of each weight stays what it is.
 `stats` collects what was measured (tag, elements, outside, max error) for the test report.
 """
 import numpy as np
@@ -24,6 +31,7 @@ from oracle.moa_oracle import prefill_masked_dense, prefill_p_rounded
 
 ATOL, RTOL = 2e-3, 1e-2
 U_BF16 = 2.0 ** -8
+MAX_FRACTION = 2.5e-4   # of the elements of a bf16 result may lie outside the stated bound against the exact oracle
 
 stats = []
 
@@ -44,7 +52,14 @@ def close_stated(out, ref, tag):
     return float(err.max())
 
 
-def close_counted(out, ref, ref_absv, tag, max_fraction=None, u=U_BF16):
+def allowed_outside(elements, max_fraction):
+    """The count a rate of max_fraction allows among `elements`, with three standard deviations of
+    counting noise and one element on top."""
+    mean = max_fraction * elements
+    return int(mean + 3.0 * mean ** 0.5 + 1.0)
+
+
+def close_counted(out, ref, ref_absv, tag, max_fraction=MAX_FRACTION, u=U_BF16):
     """Rounded weights against the exact oracle: comparison (2) of the module docstring."""
     out = out.float().cpu().double()
     ref = torch.as_tensor(np.asarray(ref.cpu() if hasattr(ref, "cpu") else ref)).double()
@@ -57,12 +72,11 @@ def close_counted(out, ref, ref_absv, tag, max_fraction=None, u=U_BF16):
     apriori = u * (ref_absv + ref.abs()) + ATOL
     bad = err > apriori
     assert not bad.any(), (tag, float(err.max()), int(bad.sum()), [int(x) for x in bad.nonzero()[0]])
-    if max_fraction is not None:
-        assert outside <= max_fraction * out.numel(), (tag, outside, out.numel(), float(err.max()))
+    assert outside <= allowed_outside(out.numel(), max_fraction), (tag, outside, out.numel(), float(err.max()))
     return outside
 
 
-def check_prefill(out, q, k, v, sm, ns, nl, tag, max_fraction=None):
+def check_prefill(out, q, k, v, sm, ns, nl, tag, max_fraction=MAX_FRACTION):
     """out, q: [B, Hq, N, D]; k, v: [B, Hkv, N, D] with Hq a multiple of Hkv; ns, nl per kv head."""
     G = q.shape[1] // k.shape[1]
     if G > 1:

@@ -85,6 +85,70 @@ def test_sparse_plan_runs_and_keeps_only_the_rings(dev):
     assert cache.cache_valid_length[0].tolist() == [[128, 256]]
 
 
+def test_generate_on_the_patched_model(dev, capsys):
+    """transformers' own ``generate`` drives the patched model, as the reference's scripts do
+    (scripts/evaluate/chat_demo.py:72, batch_inference.py:89, retrieval_evaluate.py:53): it hands over
+    its own empty cache, which the model forward replaces by a StaticCircularCache at the prompt
+    (reference modeling_llama.py:93-112) and gets back in the outputs.  Greedy tokens equal those of the
+    step-by-step loop on the same model; ``moa_verbose`` prints the cache summary when the cache is built
+    (:95-104)."""
+    from moa_amd import StaticCircularCache
+    from moa_amd.models.interface import update_model_function
+    moa = update_model_function(_hf_model(dev, 4, 2, seed=11), "lmsys/vicuna-7b-v1.5-16k")
+    plan = {"alphas": [[192.0, 256.0], [128.0, 192.0]], "betas": [[0.0, 0.0]] * 2}
+    moa.model.set_mixture_of_attention(plan, permute_head=True, moa_verbose=True, moa_max_new_token=16)
+    ids = torch.randint(0, 1000, (2, 300), generator=torch.Generator().manual_seed(3)).to(dev)
+    new = 6
+    with torch.no_grad():
+        got = moa.generate(ids, max_new_tokens=new, do_sample=False, pad_token_id=0)
+    assert got.shape == (2, 300 + new) and torch.equal(got[:, :300], ids)
+    text = capsys.readouterr().out
+    assert "Cache configuration" in text and "cache_size" in text       # moa_verbose
+    with torch.no_grad():
+        out = moa(input_ids=ids, use_cache=True)
+        cache = out.past_key_values
+        assert isinstance(cache, StaticCircularCache)
+        want = []
+        for _ in range(new):
+            nxt = out.logits[:, -1].argmax(-1, keepdim=True)
+            want.append(nxt)
+            out = moa(input_ids=nxt, past_key_values=cache, use_cache=True)
+    assert torch.equal(got[:, 300:], torch.cat(want, dim=1))
+    # a left-padded batch goes through generate as well (mask with zeros, per-row positions): the rings
+    # hold the valid tokens only
+    mask = torch.ones(2, 300, dtype=torch.int64, device=dev)
+    mask[1, :100] = 0
+    moa.model.moa_verbose = False
+    with torch.no_grad():
+        res = moa.generate(ids, attention_mask=mask, max_new_tokens=3, do_sample=False, pad_token_id=0,
+                           return_dict_in_generate=True)
+    assert res.sequences.shape == (2, 303)
+    cache = res.past_key_values
+    assert isinstance(cache, StaticCircularCache)
+    # 3 tokens generated, the last of them not yet fed back: prompt + 2 positions seen
+    assert cache.get_seq_length() == 302
+    sizes = cache.cache_max_length[0].tolist()
+    assert cache.cache_valid_length[0].tolist() == [[min(302, c) for c in sizes], [min(202, c) for c in sizes]]
+
+
+def test_model_forward_arguments(dev):
+    """return_dict=False, output_hidden_states, cache_position and output_attentions behave as in the
+    reference's model forward (modeling_llama.py:64-70,114-129,183-198)."""
+    from moa_amd.models.interface import update_model_function
+    moa = update_model_function(_hf_model(dev, 4, 4, seed=5), "llama")
+    moa.model.set_mixture_of_attention({"alphas": [[512.0] * 4] * 2, "betas": [[0.0] * 4] * 2}, last_hidden_only=False)
+    ids = torch.randint(0, 1000, (1, 130), generator=torch.Generator().manual_seed(4)).to(dev)
+    with torch.no_grad():
+        a = moa.model(input_ids=ids, use_cache=True, output_hidden_states=True)
+        assert a.last_hidden_state.shape == (1, 130, 256) and len(a.hidden_states) == 3
+        b = moa.model(input_ids=ids, use_cache=True, return_dict=False)
+        assert isinstance(b, tuple) and torch.equal(b[0], a.last_hidden_state)
+        c = moa.model(input_ids=ids, use_cache=True, cache_position=torch.arange(130, device=dev))
+        assert torch.equal(c.last_hidden_state, a.last_hidden_state)
+        with pytest.raises(NotImplementedError):
+            moa.model(input_ids=ids, output_attentions=True)
+
+
 def test_unknown_model_names_are_refused():
     from moa_amd.models.interface import update_model_function
     with pytest.raises(NotImplementedError):
