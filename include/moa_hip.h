@@ -61,6 +61,17 @@ const char* moa_last_error(void);
  * sink_blocks, local_blocks: int64 [Hkv] BLOCK counts (the reference passes
  * sink_size // 64 and local_size // 64, mixture_of_attention.py:441-442).
  * dtype: MOA_DTYPE_F16 or MOA_DTYPE_BF16.  D: 64 or 128.
+ *
+ * The launch hands its (head, query tile) work items to one resident work-group
+ * per CU through a few counters in a small device array that is part of the
+ * library's device image (64 bytes per launch, 256 slots used in turn; a slot is
+ * left cleared by the launch that used it).  The call itself allocates nothing.
+ * Launches may overlap on one GPU as long as fewer than 256 of them are under
+ * way at once.  The first call on a device looks that array up and the first
+ * call per (dtype, D) sets a kernel attribute: make one ordinary call per device
+ * and (dtype, D) before recording the call into a HIP graph; a recorded call
+ * keeps the slot it was recorded with, so replays of ONE graph that overlap each
+ * other on a GPU are not supported.
  */
 int moa_prefill_fwd(const void* q, const void* k, const void* v, void* o,
                     const int64_t* q_strides, const int64_t* k_strides,
@@ -115,6 +126,10 @@ int moa_decode_fwd(const void* q, const void* kc, const void* vc, void* o,
  * All calls on one GPU share that GPU's array: calls that may overlap on one
  * GPU (different streams, different threads) race on it and must be
  * serialised by the caller.
+ * The first call on a device looks the array's device address up and the first
+ * call of a (dtype, head_dim, grouped or not) class sets a kernel attribute:
+ * make one ordinary call per device and class before recording the call into a
+ * HIP graph.
  */
 #define MOA_DECODE_NOALLOC_MAX_BYTES (32u << 20)
 int moa_decode_fwd_noalloc(const void* q, const void* kc, const void* vc, void* o,

@@ -94,3 +94,19 @@ def test_missing_library_is_loud(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libmoa_hip.so"))
     with pytest.raises(_lib.MoaKernelError):
         _lib.load()
+
+
+def test_python_constants_match_the_header():
+    """The size limit of the entry point that allocates nothing is written down twice (header and
+    _lib.py): the two must agree."""
+    import re
+    from moa_amd import _lib
+    text = open(os.path.join(ROOT, "include", "moa_hip.h")).read()
+    m = re.search(r"#define\s+MOA_DECODE_NOALLOC_MAX_BYTES\s+\((\d+)u\s*<<\s*(\d+)\)", text)
+    assert m, "MOA_DECODE_NOALLOC_MAX_BYTES not found in the header"
+    assert int(m.group(1)) << int(m.group(2)) == _lib.MOA_DECODE_NOALLOC_MAX_BYTES
+    for name in ("MOA_OK", "MOA_ERR_ARG", "MOA_ERR_UNSUPPORTED", "MOA_ERR_LAUNCH", "MOA_ERR_WORKSPACE",
+                 "MOA_DTYPE_F16", "MOA_DTYPE_BF16", "MOA_DTYPE_F32"):
+        m = re.search(r"#define\s+%s\s+\(?(-?\d+)\)?" % name, text) or re.search(r"%s\s*=\s*(-?\d+)" % name, text)
+        assert m, name
+        assert int(m.group(1)) == getattr(_lib, name), name

@@ -115,3 +115,42 @@ def test_headline_shape_fits(dev):
     from moa_amd import _lib
     lib = _lib.load()
     assert lib.moa_decode_workspace_bytes(64, 32, 32, 128, 190_000) <= _lib.MOA_DECODE_NOALLOC_MAX_BYTES
+
+
+def test_recorded_into_a_hip_graph(dev):
+    """After one ordinary call (which does the per-device and per-kernel set-up), the entry point can be
+    recorded into a HIP graph: it allocates nothing and its scratch sits at a fixed address.  Every replay,
+    with eager work between the replays, gives the bits of the eager call."""
+    from moa_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(7)
+    q, kc, vc, hs, hv = _inputs(rng, 3, [64, 3008, 576, 1344], 4, 128, torch.bfloat16, dev, partial=True)
+    B, Hq, D = q.shape
+    Hkv, sumC = hs.shape[1], kc.shape[1]
+    hs_d, hv_d = torch.from_numpy(hs).to(dev), torch.from_numpy(hv).to(dev)
+    code = _lib.dtype_code(q.dtype)
+
+    def call(o):
+        rc = lib.moa_decode_fwd_noalloc(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), o.data_ptr(), hs_d.data_ptr(),
+                                        hv_d.data_ptr(), B, Hq, Hkv, D, sumC, D ** -0.5, code, _lib.current_stream_ptr(dev))
+        assert rc == 0, _lib.last_error()
+
+    eager = torch.empty_like(q)
+    call(eager)                       # the ordinary call that comes first
+    torch.cuda.synchronize()
+    o_graph = torch.full_like(q, float("nan"))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(o_graph)
+    for i in range(3):
+        o_graph.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(o_graph, eager), i
+        # eager work between the replays: new queries through the same scratch
+        q2 = torch.randn_like(q)
+        o2 = torch.empty_like(q)
+        rc = lib.moa_decode_fwd_noalloc(q2.data_ptr(), kc.data_ptr(), vc.data_ptr(), o2.data_ptr(), hs_d.data_ptr(),
+                                        hv_d.data_ptr(), B, Hq, Hkv, D, sumC, D ** -0.5, code, _lib.current_stream_ptr(dev))
+        assert rc == 0
+        torch.cuda.synchronize()
