@@ -61,6 +61,8 @@ def parse_args():
                     help="run moa_amd.efficiency_test (the reference's efficiency script: same modes and printed "
                          "figures) on the whole decoder of --shape at that config's batch and prompt length, "
                          "--new-tokens decode steps; not the contract line")
+    ap.add_argument("--no-e2e", action="store_true",
+                    help="skip the whole-decoder runs of the two end-to-end configurations in the default line")
     ap.add_argument("--only", choices=["decode", "prefill", "copy", "e2e", "e2e-full", "gqa"], default=None,
                     help="profiling aid: run one part only and print its figures (not the contract line)")
     return ap.parse_args()
@@ -493,6 +495,70 @@ def bench_prefill(torch, dev, args, B=4, Hq=32, Hkv=32, N=8192, iters=None, alph
     }
 
 
+def bench_prompt_side(torch, dev, iters=6):
+    """The kernels between the projections and the attention in a prompt pass, at the layer shape of the
+    7B end-to-end config (B=8, 32 heads, N=16384, D=128, bf16): the rotary embedding of q and k
+    (moa_rope_fwd) and the bulk insert of the rotated k and of v into the rings
+    (moa_cache_prefill_insert), without and with an attention mask (two batch rows left-padded).
+    Algorithmic bytes: rotary = q and k read and written once + cos and sin; insert = the rows that are
+    kept (per head min(N, cache size)) of k and of v read and written once + the ring bookkeeping."""
+    from moa_amd import StaticCircularCache
+    from moa_amd.kernels.rotary import apply_rotary_pos_emb
+    from moa_amd.models.llama.modeling_llama import rotary_cos_sin
+    from moa_amd.workloads import elastic_spans, ring_cache_sizes
+
+    B, H, N, D, dtype = 8, 32, 16384, 128, torch.bfloat16
+    gen = torch.Generator(device=dev).manual_seed(3)
+    q, k, v = (torch.randn(B, N, H, D, generator=gen, device=dev, dtype=dtype).transpose(1, 2) for _ in range(3))
+    cos, sin = rotary_cos_sin(torch.arange(N, device=dev)[None, :], D, dtype)
+    cs, ss = ring_cache_sizes(elastic_spans(H, N, seed=0))
+
+    def timed(fn, n):
+        out = []
+        for _ in range(n):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize(dev)
+            out.append(e0.elapsed_time(e1))
+        out.sort()
+        return out[len(out) // 2] * 1e3   # us
+
+    res = {"workload": f"B={B},H={H},N={N},D={D},bf16; rings = 64 sinks + elastic window (seed 0)"}
+    for _ in range(2):
+        apply_rotary_pos_emb(q, k, cos, sin)
+    rope_us = timed(lambda: apply_rotary_pos_emb(q, k, cos, sin), iters)
+    rope_bytes = 2 * (q.numel() + k.numel()) * 2 + 2 * cos.numel() * 2
+    res["rope_prefill"] = {"us": rope_us, "bytes": rope_bytes, "GB/s": rope_bytes / rope_us / 1e3,
+                           "frac_of_hbm_peak": rope_bytes / rope_us / 1e3 / HBM_PEAK_GBS,
+                           "note": "includes torch's allocation of the two outputs (caching allocator, no hipMalloc after the first call)"}
+    kept = sum(min(N, c) for c in cs)
+    ins_bytes = 2 * 2 * B * kept * D * 2 + 3 * 8 * B * H + 8 * B * sum(cs)
+    mask = torch.ones(B, N, dtype=torch.int64, device=dev)
+    mask[1, :1000] = 0
+    mask[5, :7777] = 0
+    for name, am in (("prefill_insert", None), ("prefill_insert_masked", mask)):
+        us = []
+        for i in range(iters + 1):
+            cache = StaticCircularCache([cs], batch_size=B, head_dim=D, static_size=[ss], device=dev, dtype=dtype)
+            cache._to_device(0, dev)      # the K/V allocation stays outside the timed region
+            torch.cuda.synchronize(dev)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            cache.update(k, v, 0, attention_mask=am)
+            e1.record()
+            torch.cuda.synchronize(dev)
+            if i:
+                us.append(e0.elapsed_time(e1) * 1e3)
+            del cache
+        us.sort()
+        med = us[len(us) // 2]
+        res[name] = {"us": med, "bytes": ins_bytes, "GB/s": ins_bytes / med / 1e3,
+                     "frac_of_hbm_peak": ins_bytes / med / 1e3 / HBM_PEAK_GBS}
+    return res
+
+
 def bench_prefill_c1(torch, dev, iters=20):
     """The CPU-reference configuration on the GPU kernel (fp16: the kernel has no fp32 path), to put a
     GPU time beside cpu_baseline.prefill_c1."""
@@ -552,6 +618,7 @@ def cpu_baseline(torch, args, budget_s=12.0):
     tok_s = 1.0 / (mean_layer * L)
     return {
         "prefill_c1": cpu_prefill_c1(torch),
+        "prefill_c2": cpu_prefill_c2_slice(torch),
         "append": cpu_append(torch, args),
         "value": tok_s,
         "unit": "tokens/s",
@@ -581,6 +648,29 @@ def cpu_prefill_c1(torch):
             "workload": "B=1,H=32,D=64,N=2048,fp32,sink=64,window uniform in {256..1024}: dense masked SDPA, whole config",
             "gflops_live": 4.0 * D * pairs * B / dt / 1e9,
             "gflops_dense_causal": 4.0 * D * H * B * (N * (N + 1) / 2) / dt / 1e9}
+
+
+def cpu_prefill_c2_slice(torch, heads=4):
+    """A slice of the prefill benchmark configuration (B=4, H=32, D=128, N=8192) on the host cores: ONE
+    batch row and the first `heads` heads through the oracle's dense masked attention in fp32 (the
+    arithmetic of the reference's dense path), scaled linearly to the whole configuration (the work of
+    a (batch row, head) pair on the dense path does not depend on its span)."""
+    from oracle.moa_oracle import prefill_masked_dense
+    from moa_amd.workloads import elastic_spans, prefill_work
+    B, H, N, D = 4, 32, 8192, 128
+    spans = elastic_spans(H, N, seed=0)
+    g = torch.Generator().manual_seed(7)
+    q, k, v = (torch.randn(1, heads, N, D, generator=g).to(torch.bfloat16).float() for _ in range(3))
+    ns, nl = [1] * heads, [s // 64 for s in spans[:heads]]
+    t0 = time.perf_counter()
+    prefill_masked_dense(q, k, v, D ** -0.5, ns, nl)
+    dt = time.perf_counter() - t0
+    scale = B * H / heads
+    flops_live, _, _ = prefill_work(N, [1] * H, [s // 64 for s in spans], B, D)
+    return {"seconds_slice": dt, "seconds_whole_config_scaled": dt * scale, "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"1 of {B} batch rows x {heads} of {H} heads of B=4,H=32,D=128,N=8192 (bf16 values in fp32), dense masked SDPA; "
+                      f"scaled by {scale:g} to the whole configuration",
+            "gflops_live_scaled": flops_live / (dt * scale) / 1e9}
 
 
 def cpu_append(torch, args, rows=8, steps=20):
@@ -674,6 +764,20 @@ def main():
             pre = {"error": str(e)}
     torch.cuda.empty_cache()
     gqa = bench_decode_gqa(torch, dev, args)
+    prompt_side = bench_prompt_side(torch, dev)
+    torch.cuda.empty_cache()
+    e2e = None
+    if not args.no_e2e:
+        # the two end-to-end configurations as whole decoders (prompt pass, then greedy steps, eager and
+        # replayed from a HIP graph): 7B shape with 256 steps, 70B grouped-query shape with 128
+        import argparse as _ap
+        e2e = {}
+        for key, shape, steps in (("c4_7b", "7b", 256), ("c5_70b", "70b", 128)):
+            try:
+                e2e[key] = bench_e2e_full(torch, dev, _ap.Namespace(shape=shape, new_tokens=steps))
+            except torch.cuda.OutOfMemoryError as e:   # a smaller card: say so instead of failing the line
+                e2e[key] = {"error": "out of device memory: " + str(e)[:200]}
+            torch.cuda.empty_cache()
     cpu = None if args.no_cpu else cpu_baseline(torch, args)
 
     line = {
@@ -716,6 +820,8 @@ def main():
         "rope_append": rope,
         "prefill": pre,
         "decode_gqa": gqa,
+        "prompt_side": prompt_side,
+        "e2e": e2e,
     }
     print(json.dumps(line))
 

@@ -102,6 +102,13 @@ class StaticCircularCache:
             torch.zeros((batch_size, h), dtype=torch.int64, device=device)
             for h in self.num_head_for_each_layer]
 
+    def __getstate__(self):
+        """Copies (copy.deepcopy, pickling) do not take the per-layer call arguments along: those hold
+        device addresses of THIS object's tensors."""
+        state = self.__dict__.copy()
+        state["_step_args"] = [None] * self.num_layers
+        return state
+
     # ------------------------------------------------------------------
     # layout helpers (same results as the reference's static methods)
     # ------------------------------------------------------------------
