@@ -533,12 +533,16 @@ def bench_prompt_side(torch, dev, iters=6):
     res["rope_prefill"] = {"us": rope_us, "bytes": rope_bytes, "GB/s": rope_bytes / rope_us / 1e3,
                            "frac_of_hbm_peak": rope_bytes / rope_us / 1e3 / HBM_PEAK_GBS,
                            "note": "includes torch's allocation of the two outputs (caching allocator, no hipMalloc after the first call)"}
-    kept = sum(min(N, c) for c in cs)
-    ins_bytes = 2 * 2 * B * kept * D * 2 + 3 * 8 * B * H + 8 * B * sum(cs)
     mask = torch.ones(B, N, dtype=torch.int64, device=dev)
     mask[1, :1000] = 0
     mask[5, :7777] = 0
-    for name, am in (("prefill_insert", None), ("prefill_insert_masked", mask)):
+
+    def insert_bytes(valid):   # valid tokens per batch row
+        kept = sum(min(nv, c) for nv in valid for c in cs)
+        return 2 * 2 * kept * D * 2 + 3 * 8 * B * H + 8 * kept
+
+    for name, am, ins_bytes in (("prefill_insert", None, insert_bytes([N] * B)),
+                                ("prefill_insert_masked", mask, insert_bytes(mask.sum(1).tolist()) + 8 * B * N)):
         us = []
         for i in range(iters + 1):
             cache = StaticCircularCache([cs], batch_size=B, head_dim=D, static_size=[ss], device=dev, dtype=dtype)

@@ -86,36 +86,27 @@ __device__ __forceinline__ bool keep_of(const HeadRing& g, int64_t slot, int64_t
   return (rap <= g.csz) || (slot < g.ch);
 }
 
-// Candidate r -> token t.  Without a mask only tokens that can be kept are
-// enumerated: r < csz walks the prompt's tail backwards (these have
-// rap = r+1 <= csz); r >= csz walks the first tokens (the only ones whose slot
-// can lie in the static part); any other token is a ring token older than
-// the last csz and is dropped by the keep rule.
-__device__ __forceinline__ bool candidate(const HeadRing& g, int64_t r, int S,
-                                          const int32_t* __restrict__ ap_row,
-                                          const int32_t* __restrict__ rap_row,
-                                          const int64_t* __restrict__ am_row,
-                                          int64_t& t, int64_t& slot) {
-  int64_t a, rap;
-  if (ap_row == nullptr) {
-    if (r < g.csz) {
-      t = (int64_t)S - 1 - r;
-      if (t < 0) return false;
-    } else {
-      t = r - g.csz;
-      if (t >= (int64_t)S - g.csz || t > g.s) return false;
-    }
-    a = t;
-    rap = (int64_t)S - t;
+// Candidate r -> the token with advancing position a (its index among the row's valid tokens; without a
+// mask every token is valid and a is the token's position).  Only tokens that can be kept are
+// enumerated: r < csz walks the valid tokens from the last one backwards (these have
+// rap = r+1 <= csz); r >= csz walks the first ones (the only ones whose slot can lie in the static
+// part); any other token is a ring token older than the last csz and is dropped by the keep rule.
+// n_valid: valid tokens of the batch row.  Returns whether the candidate is kept, with a and its slot.
+__device__ __forceinline__ bool candidate(const HeadRing& g, int64_t r, int64_t n_valid, int64_t& a, int64_t& slot) {
+  if (r < g.csz) {
+    a = n_valid - 1 - r;
+    if (a < 0) return false;
   } else {
-    t = r;
-    if (t >= S) return false;
-    if (am_row[t] != 1) return false;
-    a = ap_row[t];
-    rap = rap_row[t];
+    a = r - g.csz;
+    if (a >= n_valid - g.csz || a > g.s) return false;
   }
+  const int64_t rap = n_valid - a;   // valid tokens at or after this one (:1081-1086)
   slot = slot_of(g, a);
   return keep_of(g, slot, rap);
+}
+// how many candidates a head has
+__device__ __forceinline__ int64_t candidate_count(const HeadRing& g, int64_t n_valid) {
+  return min(n_valid, g.csz + g.s + 1);
 }
 
 __device__ __forceinline__ HeadRing load_ring(const int64_t* update_index, const int64_t* circ_head,
@@ -130,49 +121,45 @@ __device__ __forceinline__ HeadRing load_ring(const int64_t* update_index, const
   return g;
 }
 
-// ap[b, t] = (#ones in am[b, 0..t]) - 1 for t in [0, S), ap[b, S] = ap[b, S-1] + 1;
-// rap[b, t] = #ones in am[b, t..S-1]   (:1075-1086)
-__global__ __launch_bounds__(256) void mask_scan_kernel(const int64_t* __restrict__ am,
-                                                         int64_t am_stride, int S,
-                                                         int32_t* __restrict__ ap,
-                                                         int32_t* __restrict__ rap) {
-  __shared__ int32_t part[256];
+// With an attention mask: the positions of a batch row's valid tokens (mask == 1) in order,
+// tok_of[b, a] = position of the a-th valid token, and their number n_valid[b].  This is the inverse of
+// the reference's advancing_pos = cumsum(mask) - 1 (:1075-1080); its reversed_advancing_pos of a valid
+// token is n_valid - a (:1081-1086).  One work-group per batch row walks the row in slices of its size:
+// coalesced loads, a ballot and a population count inside each wave, the waves' totals through LDS.
+constexpr int kScanThreads = 1024;
+__global__ __launch_bounds__(kScanThreads) void mask_compact_kernel(const int64_t* __restrict__ am,
+                                                                     int64_t am_stride, int S,
+                                                                     int32_t* __restrict__ tok_of,
+                                                                     int32_t* __restrict__ n_valid) {
+  constexpr int kWaves = kScanThreads / 64;
+  __shared__ int s_wave[kWaves];
   const int b = blockIdx.x;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t* row = am + (int64_t)b * am_stride;
-  const int per = (S + 255) / 256;
-  const int t0 = tid * per;
-  const int t1 = min(S, t0 + per);
-  int32_t sum = 0;
-  for (int t = t0; t < t1; ++t) sum += (int32_t)row[t];
-  part[tid] = sum;
-  __syncthreads();
-  if (tid == 0) {
-    int32_t run = 0;
-    for (int i = 0; i < 256; ++i) {
-      int32_t x = part[i];
-      part[i] = run;
-      run += x;
+  int32_t* out = tok_of + (int64_t)b * S;
+  int base = 0;
+  for (int t0 = 0; t0 < S; t0 += kScanThreads) {
+    const int t = t0 + tid;
+    const bool valid = t < S && row[t] == 1;
+    const unsigned long long bal = __ballot(valid);
+    const int before = __popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) s_wave[wave] = __popcll(bal);
+    __syncthreads();
+    int off = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const int c = s_wave[w];
+      off += (w < wave) ? c : 0;
+      total += c;
     }
+    if (valid) out[base + off + before] = t;
+    base += total;
+    __syncthreads();   // s_wave is written again in the next slice
   }
-  __syncthreads();
-  int32_t total = part[255];
-  {
-    // total = exclusive prefix of the last thread + its own sum
-    const int lt0 = 255 * per;
-    for (int t = lt0; t < S; ++t) total += (int32_t)row[t];
-  }
-  int32_t run = part[tid];
-  int32_t* ap_row = ap + (int64_t)b * (S + 1);
-  int32_t* rap_row = rap + (int64_t)b * S;
-  for (int t = t0; t < t1; ++t) {
-    const int32_t x = (int32_t)row[t];
-    run += x;
-    ap_row[t] = run - 1;
-    rap_row[t] = total - run + x;
-  }
-  if (tid == 0) ap_row[S] = total;  // ap[S-1] + 1 == total - 1 + 1
+  if (tid == 0) n_valid[b] = base;
 }
+
+constexpr int kRowsPerThread = 4;   // rows a group of 16 lanes moves: all loads go out before the first store
 
 __global__ __launch_bounds__(kCacheThreads) void cache_prefill_copy_kernel(
     const char* __restrict__ k, const char* __restrict__ v,
@@ -180,26 +167,47 @@ __global__ __launch_bounds__(kCacheThreads) void cache_prefill_copy_kernel(
     char* __restrict__ kc, char* __restrict__ vc, int64_t* __restrict__ mask_cache,
     const int64_t* __restrict__ update_index, const int64_t* __restrict__ circ_head,
     const int64_t* __restrict__ circ_size, const int64_t* __restrict__ static_size,
-    const int64_t* __restrict__ am, int64_t am_stride, const int32_t* __restrict__ ap,
-    const int32_t* __restrict__ rap, int64_t kv_len, int H, int S, int row_bytes, int64_t sumC) {
+    const int32_t* __restrict__ tok_of, const int32_t* __restrict__ n_valid, int64_t kv_len, int H, int S,
+    int row_bytes, int64_t sumC) {
   const int lane = threadIdx.x % kRowLanes;
-  const int64_t r = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kRowLanes;
   const int h = blockIdx.y;
   const int b = blockIdx.z;
   const int64_t bh = (int64_t)b * H + h;
   const HeadRing g = load_ring(update_index, circ_head, circ_size, static_size, kv_len, bh, h);
-  int64_t t, slot;
-  const bool keep = candidate(g, r, S, ap ? ap + (int64_t)b * (S + 1) : nullptr,
-                              rap ? rap + (int64_t)b * S : nullptr,
-                              am ? am + (int64_t)b * am_stride : nullptr, t, slot);
-  if (!keep || slot < 0 || slot >= sumC) return;
-  if (kc != nullptr) {
-    const int units = row_bytes / 16;
-    const size_t dst = ((size_t)b * sumC + slot) * row_bytes;
-    copy_row16(k + b * k_sb + h * k_sh + t * k_ss, kc + dst, units, lane);
-    copy_row16(v + b * v_sb + h * v_sh + t * v_ss, vc + dst, units, lane);
+  const int64_t nv = n_valid ? (int64_t)n_valid[b] : (int64_t)S;
+  const int64_t r0 = (int64_t)blockIdx.x * (kRowsPerBlock * kRowsPerThread) + threadIdx.x / kRowLanes;
+  if ((int64_t)blockIdx.x * (kRowsPerBlock * kRowsPerThread) >= candidate_count(g, nv)) return;
+  const char* src_k[kRowsPerThread];
+  const char* src_v[kRowsPerThread];
+  size_t dst[kRowsPerThread];
+  bool keep[kRowsPerThread];
+#pragma unroll
+  for (int j = 0; j < kRowsPerThread; ++j) {
+    int64_t a, slot;
+    keep[j] = candidate(g, r0 + j * kRowsPerBlock, nv, a, slot) && slot >= 0 && slot < sumC;
+    const int64_t t = keep[j] ? (tok_of ? (int64_t)tok_of[(int64_t)b * S + a] : a) : 0;
+    src_k[j] = k + b * k_sb + h * k_sh + t * k_ss;
+    src_v[j] = v + b * v_sb + h * v_sh + t * v_ss;
+    dst[j] = keep[j] ? ((size_t)b * sumC + slot) * row_bytes : 0;
+    if (keep[j] && lane == 0 && mask_cache != nullptr) mask_cache[(size_t)b * sumC + slot] = 1;
   }
-  if (lane == 0 && mask_cache != nullptr) mask_cache[(size_t)b * sumC + slot] = 1;
+  if (kc == nullptr) return;
+  const int units = row_bytes / 16;
+  for (int u = lane; u < units; u += kRowLanes) {
+    u32x4 xk[kRowsPerThread], xv[kRowsPerThread];
+#pragma unroll
+    for (int j = 0; j < kRowsPerThread; ++j)
+      if (keep[j]) {
+        xk[j] = *reinterpret_cast<const u32x4*>(src_k[j] + (size_t)u * 16);
+        xv[j] = *reinterpret_cast<const u32x4*>(src_v[j] + (size_t)u * 16);
+      }
+#pragma unroll
+    for (int j = 0; j < kRowsPerThread; ++j)
+      if (keep[j]) {
+        *reinterpret_cast<u32x4*>(kc + dst[j] + (size_t)u * 16) = xk[j];
+        *reinterpret_cast<u32x4*>(vc + dst[j] + (size_t)u * 16) = xv[j];
+      }
+  }
 }
 
 // One wavefront per (b, h): count the kept tokens, then move the pointers
@@ -208,8 +216,7 @@ __global__ __launch_bounds__(kCacheThreads) void cache_prefill_copy_kernel(
 __global__ __launch_bounds__(256) void cache_prefill_index_kernel(
     int64_t* __restrict__ update_index, int64_t* __restrict__ valid_len,
     const int64_t* __restrict__ circ_head, const int64_t* __restrict__ circ_size,
-    const int64_t* __restrict__ static_size, const int64_t* __restrict__ am, int64_t am_stride,
-    const int32_t* __restrict__ ap, const int32_t* __restrict__ rap, int64_t kv_len, int B, int H,
+    const int64_t* __restrict__ static_size, const int32_t* __restrict__ n_valid, int64_t kv_len, int B, int H,
     int S) {
   const int lane = threadIdx.x & 63;
   const int64_t bh = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -217,20 +224,16 @@ __global__ __launch_bounds__(256) void cache_prefill_index_kernel(
   const int b = (int)(bh / H);
   const int h = (int)(bh % H);
   const HeadRing g = load_ring(update_index, circ_head, circ_size, static_size, kv_len, bh, h);
-  const int32_t* ap_row = ap ? ap + (int64_t)b * (S + 1) : nullptr;
-  const int32_t* rap_row = rap ? rap + (int64_t)b * S : nullptr;
-  const int64_t* am_row = am ? am + (int64_t)b * am_stride : nullptr;
-  // number of candidates: all tokens with a mask; else tail (<= csz) + first s+1 tokens
-  const int64_t n_cand = ap ? (int64_t)S : min((int64_t)S, g.csz + g.s + 1);
+  const int64_t nv = n_valid ? (int64_t)n_valid[b] : (int64_t)S;
+  const int64_t n_cand = candidate_count(g, nv);
   int count = 0;
   for (int64_t r = lane; r < n_cand; r += 64) {
-    int64_t t, slot;
-    count += candidate(g, r, S, ap_row, rap_row, am_row, t, slot) ? 1 : 0;
+    int64_t a, slot;
+    count += candidate(g, r, nv, a, slot) ? 1 : 0;
   }
   for (int off = 32; off > 0; off >>= 1) count += __shfl_xor(count, off, 64);
   if (lane == 0) {
-    const int64_t a_end = ap ? (int64_t)ap_row[S] : (int64_t)S;
-    update_index[bh] = slot_of(g, a_end);
+    update_index[bh] = slot_of(g, nv);   // the slot the token after the last valid one would take (:1110)
     valid_len[bh] += count;
   }
 }
@@ -323,37 +326,35 @@ extern "C" int moa_cache_prefill_insert(const void* k, const void* v, const int6
     for (int i = 0; i < 3; ++i) { ks[i] = k_strides[i] * eb; vs[i] = v_strides[i] * eb; }
   }
   hipStream_t st = (hipStream_t)stream;
-  int32_t* ap = nullptr;
-  int32_t* rap = nullptr;
-  int64_t n_rows;
+  int32_t* tok_of = nullptr;
+  int32_t* n_valid = nullptr;
   if (attention_mask != nullptr) {
     const size_t need = moa_cache_prefill_workspace_bytes(B, S);
     if (workspace == nullptr || workspace_bytes < need)
       return fail(MOA_ERR_WORKSPACE, "moa_cache_prefill_insert: workspace %zu < %zu bytes", workspace_bytes, need);
-    ap = reinterpret_cast<int32_t*>(workspace);
-    rap = ap + (size_t)B * ((size_t)S + 1);
-    hipLaunchKernelGGL(mask_scan_kernel, dim3(B), dim3(256), 0, st, attention_mask, am_stride, S, ap, rap);
+    tok_of = reinterpret_cast<int32_t*>(workspace);
+    n_valid = tok_of + (size_t)B * (size_t)S;
+    hipLaunchKernelGGL(mask_compact_kernel, dim3(B), dim3(kScanThreads), 0, st, attention_mask, am_stride, S, tok_of,
+                       n_valid);
     int rc = check_launch("moa_cache_prefill_insert(mask scan)");
     if (rc) return rc;
-    n_rows = S;
-  } else {
-    // candidates r >= S never name a token (see candidate())
-    n_rows = S;
-    if (max_cache_size > 0 && max_cache_size + 1 < n_rows) n_rows = max_cache_size + 1;
   }
+  // candidates r >= S never name a token, nor do those past a head's cache size + 1 (see candidate())
+  int64_t n_rows = S;
+  if (max_cache_size > 0 && max_cache_size + 1 < n_rows) n_rows = max_cache_size + 1;
   if (kc != nullptr || mask_cache != nullptr) {
-    dim3 grid((unsigned)((n_rows + kRowsPerBlock - 1) / kRowsPerBlock), (unsigned)H, (unsigned)B);
+    constexpr int kPerBlock = kRowsPerBlock * kRowsPerThread;
+    dim3 grid((unsigned)((n_rows + kPerBlock - 1) / kPerBlock), (unsigned)H, (unsigned)B);
     hipLaunchKernelGGL(cache_prefill_copy_kernel, grid, dim3(kCacheThreads), 0, st, (const char*)k,
                        (const char*)v, ks[0], ks[1], ks[2], vs[0], vs[1], vs[2], (char*)kc, (char*)vc,
                        mask_cache, (const int64_t*)update_index, circ_head, circ_size, static_size,
-                       attention_mask, am_stride, (const int32_t*)ap, (const int32_t*)rap, kv_len, H, S,
-                       D * eb, sumC);
+                       (const int32_t*)tok_of, (const int32_t*)n_valid, kv_len, H, S, D * eb, sumC);
     int rc = check_launch("moa_cache_prefill_insert(copy)");
     if (rc) return rc;
   }
   const int64_t n = (int64_t)B * H;
   hipLaunchKernelGGL(cache_prefill_index_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, st,
-                     update_index, valid_len, circ_head, circ_size, static_size, attention_mask,
-                     am_stride, (const int32_t*)ap, (const int32_t*)rap, kv_len, B, H, S);
+                     update_index, valid_len, circ_head, circ_size, static_size, (const int32_t*)n_valid, kv_len, B, H,
+                     S);
   return check_launch("moa_cache_prefill_insert(index)");
 }

@@ -117,22 +117,33 @@ struct RopeTensor {
   int64_t db, dh, dn;   // destination byte strides
 };
 
-// q and k of a whole prompt (or of one step): one thread per chunk pair.
+// q and k of a whole prompt (or of one step): one thread per chunk pair.  Consecutive threads walk a row,
+// then the dimension in which the SOURCE rows lie closer together (heads for views of [B, N, H, D]
+// projections, tokens for [B, H, N, D] tensors), so that a wave reads one consecutive piece of memory.
 template <typename E>
 __global__ __launch_bounds__(kRopeThreads) void rope_kernel(RopeTensor tq, RopeTensor tk,
                                                              const char* __restrict__ cos,
                                                              const char* __restrict__ sin, int64_t cs_sb,
                                                              int64_t cs_sn, int B, int Hq, int Hkv, int N,
-                                                             int pairs_per_row, int half_bytes) {
+                                                             int pairs_per_row, int half_bytes, bool heads_inner) {
   const int64_t idx = (int64_t)blockIdx.x * kRopeThreads + threadIdx.x;
   const int64_t total = (int64_t)B * (Hq + Hkv) * N * pairs_per_row;
   if (idx >= total) return;
   const int pair = (int)(idx % pairs_per_row);
   int64_t row = idx / pairs_per_row;
-  const int n = (int)(row % N);
-  row /= N;
-  const int hh = (int)(row % (Hq + Hkv));
-  const int b = (int)(row / (Hq + Hkv));
+  int n, hh;
+  if (heads_inner) {
+    hh = (int)(row % (Hq + Hkv));
+    row /= (Hq + Hkv);
+    n = (int)(row % N);
+    row /= N;
+  } else {
+    n = (int)(row % N);
+    row /= N;
+    hh = (int)(row % (Hq + Hkv));
+    row /= (Hq + Hkv);
+  }
+  const int b = (int)row;
   const bool is_q = hh < Hq;
   const RopeTensor& t = is_q ? tq : tk;
   const int h = is_q ? hh : hh - Hq;
@@ -254,9 +265,11 @@ extern "C" int moa_rope_fwd(const void* q, const void* k, void* q_out, void* k_o
   if (blocks > 0x7fffffffLL) return fail(MOA_ERR_UNSUPPORTED, "%s: too many rows", who);
   hipStream_t st = (hipStream_t)stream;
   const int64_t csb = cs_strides[0] * eb, csn = cs_strides[1] * eb;
+  const RopeTensor& lead = Hq > 0 ? tq : tk;
+  const bool heads_inner = lead.sh < lead.sn;
 #define MOA_ROPE_LAUNCH(E)                                                                                  \
   hipLaunchKernelGGL(rope_kernel<E>, dim3((unsigned)blocks), dim3(kRopeThreads), 0, st, tq, tk,             \
-                     (const char*)cos, (const char*)sin, csb, csn, B, Hq, Hkv, N, pairs, half_bytes)
+                     (const char*)cos, (const char*)sin, csb, csn, B, Hq, Hkv, N, pairs, half_bytes, heads_inner)
   if (dtype == MOA_DTYPE_F16) MOA_ROPE_LAUNCH(EF16);
   else if (dtype == MOA_DTYPE_BF16) MOA_ROPE_LAUNCH(EBF16);
   else MOA_ROPE_LAUNCH(EF32);

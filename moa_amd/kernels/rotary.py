@@ -35,7 +35,10 @@ def apply_rotary_pos_emb(q: Optional[Tensor], k: Optional[Tensor], cos: Tensor, 
 
     q ``[batch, q_heads, seq_len, head_dim]``, k ``[batch, kv_heads, seq_len, head_dim]`` (any strides
     with a contiguous last dim), cos/sin ``[batch or 1, seq_len, head_dim]`` in the same dtype.
-    Returns new contiguous tensors.  Only ``unsqueeze_dim=1`` (heads in dim 1) is covered.
+    Returns new tensors laid out like their inputs when those are dense (a transposed view of a
+    ``[batch, seq_len, heads, head_dim]`` projection gives a result with the same strides, as torch's
+    elementwise evaluation of the formula does: both sides of the kernel then stream through memory),
+    contiguous otherwise.  Only ``unsqueeze_dim=1`` (heads in dim 1) is covered.
     """
     if unsqueeze_dim != 1:
         raise NotImplementedError("apply_rotary_pos_emb: only unsqueeze_dim=1 ([batch, heads, seq, dim]) is covered")
@@ -52,7 +55,7 @@ def apply_rotary_pos_emb(q: Optional[Tensor], k: Optional[Tensor], cos: Tensor, 
             outs.append(None)
             continue
         assert t.dim() == 4 and t.shape[0] == B and t.shape[2] == N and t.shape[3] == D and t.dtype == ref.dtype
-        outs.append(torch.empty(t.shape, dtype=t.dtype, device=t.device))
+        outs.append(torch.empty_like(t))   # keeps the strides of a dense input, contiguous otherwise
     qi = q if q is None or q.stride(-1) == 1 else q.contiguous()
     ki = k if k is None or k.stride(-1) == 1 else k.contiguous()
     lib = _lib.load()

@@ -43,8 +43,13 @@ def test_rope_fwd_bit_exact(dev, dtype, D):
     pos = torch.arange(N)[None, :] + torch.tensor([[0], [1000]])
     cos, sin = rope_cos_sin(pos, D, dtype=dtype)
     qe, ke = apply_rotary_pos_emb(q.to(dev), k.to(dev), cos.to(dev), sin.to(dev))
-    assert qe.shape == q.shape and ke.shape == k.shape and qe.is_contiguous()
+    # the result keeps the layout of a dense input (as torch's elementwise evaluation does)
+    assert qe.shape == q.shape and ke.shape == k.shape and qe.stride() == q.stride() and ke.stride() == k.stride()
     assert _same_bits(qe, rope_reference(q, cos, sin))
+    # contiguous [B, H, N, D] inputs (the kernel then walks tokens before heads)
+    qc, kc = q.contiguous(), k.contiguous()
+    qe2, ke2 = apply_rotary_pos_emb(qc.to(dev), kc.to(dev), cos.to(dev), sin.to(dev))
+    assert qe2.is_contiguous() and _same_bits(qe2, rope_reference(q, cos, sin)) and _same_bits(ke2, rope_reference(k, cos, sin))
     assert _same_bits(ke, rope_reference(k, cos, sin))
     # one shared position table (batch 1) broadcasts; k alone
     cos1, sin1 = cos[:1], sin[:1]
