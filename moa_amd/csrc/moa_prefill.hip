@@ -91,9 +91,24 @@ struct PrefillArgs {
   const int64_t *sink_blocks, *local_blocks;
   PrefillQueue* queue;
   int BH, Hq, group, N, n_qtiles;
+  int per_head, Hkv;   // (BH / Hq) * group pairs per kv head in the sorted list; Hq / group
   float scale_log2_signed;
 };
 typedef const PrefillArgs __attribute__((address_space(4)))* PrefillArgsPtr;
+
+// x / d and x % d for 0 <= x < 2^22, 0 < d < 2^22, through the float reciprocal and one correction step
+// each way (the compiler's general 32-bit division is four times as many instructions, and thread 0 does
+// a dozen of these per work item on the critical path).
+struct DivMod {
+  int q, r;
+};
+__device__ __forceinline__ DivMod divmod_small(int x, int d) {
+  int q = (int)((float)x * __builtin_amdgcn_rcpf((float)d));
+  int r = x - q * d;
+  if (r < 0) { q -= 1; r += d; }
+  if (r >= d) { q += 1; r -= d; }
+  return {q, r};
+}
 
 template <typename T, int D>
 __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_kernarg) {
@@ -157,13 +172,16 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
   //   [8,9] K base  [10,11] V base  [12,13] Q base (row 0 of the head)  [14,15] O base
   const int my_xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7;   // XCC_ID
   __shared__ __attribute__((aligned(16))) int s_item[2][16];
-  unsigned pre = 0;          // thread 0: the answer to the request that is under way
+  unsigned pre = 0;          // thread 0: the answer to the request that is under way, if one is (have_pre)
+  bool have_pre = true;
   bool own_alive = true;     // thread 0: the own list still had items when last asked
+  constexpr unsigned kQueueMargin = 32;   // work-groups that share a list: no tickets in advance among its last items
   auto take = [&](int slot) __attribute__((always_inline)) {
     PrefillArgsPtr ap = a0;
     asm volatile("" : "+s"(ap));
-    const int BH = ap->BH, Hq = ap->Hq, group = ap->group, N = ap->N, n_qtiles = ap->n_qtiles;
-    const int full_rounds = BH / 8, rem = BH % 8;
+    const int BH = ap->BH, group = ap->group, N = ap->N, n_qtiles = ap->n_qtiles;
+    const int per_head = ap->per_head, Hkv = ap->Hkv;
+    const int full_rounds = BH >> 3, rem = BH & 7;
     auto list_items = [&](int x) __attribute__((always_inline)) {
       const int snake = (full_rounds & 1) ? 7 - x : x;
       return (unsigned)((full_rounds + (snake < rem ? 1 : 0)) * n_qtiles);
@@ -171,7 +189,7 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
     int list = -1;
     unsigned sq = 0;
     if (own_alive) {
-      sq = pre;
+      sq = have_pre ? pre : atomicAdd(&ap->queue->next[my_xcd], 1u);
       if (sq < list_items(my_xcd)) list = my_xcd; else own_alive = false;
     }
     if (list < 0) {
@@ -181,20 +199,39 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
         if (sq < list_items(x)) { list = x; break; }
       }
     }
-    if (own_alive) pre = atomicAdd(&ap->queue->next[my_xcd], 1u);
+    // The request for the ticket after this one goes out now, so that its answer is there when it is
+    // needed -- but only while the own list is long: a ticket asked for in advance is an item this
+    // work-group is bound to, and near the end of the launch those decide how evenly the CUs finish.
+    have_pre = own_alive && sq + 1 + kQueueMargin < list_items(my_xcd);
+    if (have_pre) pre = atomicAdd(&ap->queue->next[my_xcd], 1u);
     int* d = s_item[slot];
     if (list < 0) { d[0] = -1; return; }
     const int nb = (N + kKV - 1) / kKV;
-    const int Hkv = Hq / group;
     const bool sorted = Hkv <= kMaxSortedHeads;
-    const int round = (int)sq / n_qtiles;                           // the list's round-th pair
+    // A list walks its pairs one after the other, late (long) query tiles first, and leaves the first
+    // n_last query tiles of every pair (causality keeps those short: query tile t sees at most 4 t + 4 key
+    // tiles) for the end, longest first across the pairs: heads differ little in span, so without them the
+    // last items handed out are as long as any and the CUs finish up to one whole item apart.
+    const int n_last = min(8, n_qtiles >> 2);
+    const int n_main = n_qtiles - n_last;
+    const int rounds = full_rounds + ((((full_rounds & 1) ? 7 - list : list) < rem) ? 1 : 0);
+    int round, qt;
+    if ((int)sq < rounds * n_main) {
+      const DivMod dm = divmod_small((int)sq, n_main);
+      round = dm.q;
+      qt = n_qtiles - 1 - dm.r;
+    } else {
+      const DivMod dm = divmod_small((int)sq - rounds * n_main, rounds);
+      qt = n_last - 1 - dm.q;
+      round = dm.r;
+    }
     const int pos = round * 8 + ((round & 1) ? 7 - list : list);   // position in the sorted list
     // sorted list: kv heads by rank; per kv head, batch-major, then the query heads of its group
-    const int per_head = (BH / Hq) * group;
-    const int hk = sorted ? s_head_of_rank[pos / per_head] : pos / per_head;
-    const int b = (pos % per_head) / group;
-    const int hq = hk * group + pos % group;
-    const int qt = n_qtiles - 1 - ((int)sq % n_qtiles);
+    const DivMod ph = divmod_small(pos, per_head);   // (kv head rank, place inside the head's pairs)
+    const DivMod bg = divmod_small(ph.r, group);     // (batch row, query head inside the group)
+    const int hk = sorted ? s_head_of_rank[ph.q] : ph.q;
+    const int b = bg.q;
+    const int hq = hk * group + bg.r;
     const int ns = sorted ? s_ns[hk] : (int)max((int64_t)0, min((int64_t)nb, ap->sink_blocks[hk]));
     const int nl = sorted ? s_nl[hk] : (int)max((int64_t)0, min((int64_t)nb, ap->local_blocks[hk]));
     const int mb0 = kQBlocks * qt;                              // first query block of the group
@@ -211,7 +248,11 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
     // the same K/V tile at the same step and share it in L2.  The order is free: online softmax
     // does not care, liveness and the causal mask go by tile index.
     const int n_band = n_tiles - n_sink;
-    const int band_rot = n_band > 0 ? (n_band - lo2 % n_band) % n_band : 0;
+    int band_rot = 0;
+    if (n_band > 0) {
+      band_rot = n_band - divmod_small(lo2, n_band).r;   // in [1, n_band]
+      if (band_rot == n_band) band_rot = 0;
+    }
     d[0] = n_tiles; d[1] = qt; d[2] = ns; d[3] = nl; d[4] = lo2; d[5] = n_sink; d[6] = n_band; d[7] = band_rot;
     const uint64_t kb = (uint64_t)(ap->k + b * ap->ks.b + hk * ap->ks.h);
     const uint64_t vb = (uint64_t)(ap->v + b * ap->vs.b + hk * ap->vs.h);
@@ -294,6 +335,19 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
   auto live_tile = [&](int j) __attribute__((always_inline)) { return wave_has_rows && (j <= w_hi1 || (j >= w_lo2 && j <= mbw)); };
   const int row0 = it.qt * kQRows + wave * kWRows;            // first query row of this wave
   const int64_t m_glob = row0 + mcol;                          // this lane's query row
+
+  // the Q rows are asked for first: theirs is the longest way (the other loads of an item were started by
+  // the item before it)
+  u32x4 qf[KS];              // Q fragment (B operand): Q[m][16*ks + 8*g .. +7]
+  if (n_tiles > 0) {
+    const uint16_t* qrow = it.qbase + m_glob * qs_n + 8 * g;
+    const bool ok = m_glob < N;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      u32x4 z = {0, 0, 0, 0};
+      qf[s] = ok ? *reinterpret_cast<const u32x4*>(qrow + 16 * s) : z;
+    }
+  }
 
   // ---- async tile copies: wave w, copy i fills chunks [(w*LPW+i)*64, +64) of a stage --------
   const uint16_t* const kbase = it.kbase;   // uniform
@@ -386,17 +440,6 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
     continue;
   }
   if (!prefetched) start_copies(it, rst);
-  u32x4 qf[KS];              // Q fragment (B operand): Q[m][16*ks + 8*g .. +7]
-  {
-    const uint16_t* qrow = it.qbase + m_glob * qs_n + 8 * g;
-    const bool ok = m_glob < N;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      u32x4 z = {0, 0, 0, 0};
-      qf[s] = ok ? *reinterpret_cast<const u32x4*>(qrow + 16 * s) : z;
-      qf[s] ^= u32x4{q_sign, q_sign, q_sign, q_sign};
-    }
-  }
   // the item after this one: thread 0 works its descriptor out while the loads above travel; every wave sees
   // it after this item's first barrier
   if (threadIdx.x == 0) take(par ^ 1);
@@ -614,7 +657,10 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
   // vmcnt(0) wait at their first use inside the loop, where it would also wait for the copies
 #pragma unroll
   for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[s]));
+#pragma unroll
+  for (int s = 0; s < KS; ++s) qf[s] ^= u32x4{q_sign, q_sign, q_sign, q_sign};
   asm volatile("" : "+v"(q_touch));   // the touch of the previous pass has landed as well
+  asm volatile("" : "+v"(pre));       // and so has the answer to thread 0's ticket request: its next use waits for nothing
   phase_barrier();               // K(0..2) and V(0..1) are in LDS; the next ticket is in s_ticket
   iteration(0, IC<1>{});   // no P.V yet (and no V stage to read)
   for (int t = 1; t < n_tiles; ++t) iteration(t, IC<0>{});
@@ -731,7 +777,8 @@ static int launch_prefill(const void* q, const void* k, const void* v, void* o, 
   const int n_qtiles = (N + kQRows - 1) / kQRows;
   const int BH = B * Hq;
   const int64_t items = (int64_t)BH * n_qtiles;
-  if (items > 0x7fffffffLL) return fail(MOA_ERR_UNSUPPORTED, "moa_prefill_fwd: too many work items");
+  // the queue's ticket arithmetic (divmod_small) is exact below 2^22 per list of an XCD
+  if (items > (1LL << 25) || N > (1 << 28)) return fail(MOA_ERR_UNSUPPORTED, "moa_prefill_fwd: too many work items");
   // the async copies address a tile row through a 32-bit element offset
   if (64 * ks[2] + D >= (1ll << 31) || 64 * vs[2] + D >= (1ll << 31))
     return fail(MOA_ERR_UNSUPPORTED, "moa_prefill_fwd: k/v token stride too large");
@@ -750,6 +797,7 @@ static int launch_prefill(const void* q, const void* k, const void* v, void* o, 
   args.qs = sq; args.ks = sk; args.vs = sv; args.os = so;
   args.sink_blocks = sink_blocks; args.local_blocks = local_blocks; args.queue = queue;
   args.BH = BH; args.Hq = Hq; args.group = Hq / Hkv; args.N = N; args.n_qtiles = n_qtiles;
+  args.per_head = B * (Hq / Hkv); args.Hkv = Hkv;
   args.scale_log2_signed = mfma_softmax_scale(sm_scale);
   hipLaunchKernelGGL((prefill_kernel<T, D>), dim3((unsigned)groups), dim3(NW * 64), lds, st, args);
   return check_launch("moa_prefill_fwd");
