@@ -166,16 +166,15 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
   uint32_t q_touch = 0;              // landing place of the load that pulls the next item's Q rows into L2
 
   // ---- the work queue ---------------------------------------------------------------------------
-  // Thread 0 takes tickets (one request for the own XCD's list is always under way), turns a ticket into an
-  // item descriptor once and leaves it in LDS; every wave reads it from there.
+  // Thread 0 takes a ticket for the item after the one under way (from the own XCD's list while that has
+  // items, from the other lists then; never more than that one item in advance: items bound to a work-group
+  // early spread the items that run at the same time over more of a head's keys and cost L2 hits), turns it
+  // into an item descriptor once and leaves it in LDS; every wave reads it from there.
   //   [0] n_tiles (-1: no more items)  [1] query tile  [2] ns  [3] nl  [4] lo2  [5] n_sink  [6] n_band  [7] band_rot
   //   [8,9] K base  [10,11] V base  [12,13] Q base (row 0 of the head)  [14,15] O base
   const int my_xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7;   // XCC_ID
   __shared__ __attribute__((aligned(16))) int s_item[2][16];
-  unsigned pre = 0;          // thread 0: the answer to the request that is under way, if one is (have_pre)
-  bool have_pre = true;
   bool own_alive = true;     // thread 0: the own list still had items when last asked
-  constexpr unsigned kQueueMargin = 32;   // work-groups that share a list: no tickets in advance among its last items
   auto take = [&](int slot) __attribute__((always_inline)) {
     PrefillArgsPtr ap = a0;
     asm volatile("" : "+s"(ap));
@@ -189,7 +188,7 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
     int list = -1;
     unsigned sq = 0;
     if (own_alive) {
-      sq = have_pre ? pre : atomicAdd(&ap->queue->next[my_xcd], 1u);
+      sq = atomicAdd(&ap->queue->next[my_xcd], 1u);
       if (sq < list_items(my_xcd)) list = my_xcd; else own_alive = false;
     }
     if (list < 0) {
@@ -199,11 +198,6 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
         if (sq < list_items(x)) { list = x; break; }
       }
     }
-    // The request for the ticket after this one goes out now, so that its answer is there when it is
-    // needed -- but only while the own list is long: a ticket asked for in advance is an item this
-    // work-group is bound to, and near the end of the launch those decide how evenly the CUs finish.
-    have_pre = own_alive && sq + 1 + kQueueMargin < list_items(my_xcd);
-    if (have_pre) pre = atomicAdd(&ap->queue->next[my_xcd], 1u);
     int* d = s_item[slot];
     if (list < 0) { d[0] = -1; return; }
     const int nb = (N + kKV - 1) / kKV;
@@ -262,10 +256,7 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
     d[12] = (int)(uint32_t)qb; d[13] = (int)(uint32_t)(qb >> 32); d[14] = (int)(uint32_t)ob; d[15] = (int)(uint32_t)(ob >> 32);
   };
   __syncthreads();   // the sorted heads
-  if (threadIdx.x == 0) {
-    pre = atomicAdd(&a0->queue->next[my_xcd], 1u);
-    take(0);
-  }
+  if (threadIdx.x == 0) take(0);
   __syncthreads();
 
   // An item as the waves see it.
@@ -660,7 +651,6 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
 #pragma unroll
   for (int s = 0; s < KS; ++s) qf[s] ^= u32x4{q_sign, q_sign, q_sign, q_sign};
   asm volatile("" : "+v"(q_touch));   // the touch of the previous pass has landed as well
-  asm volatile("" : "+v"(pre));       // and so has the answer to thread 0's ticket request: its next use waits for nothing
   phase_barrier();               // K(0..2) and V(0..1) are in LDS; the next ticket is in s_ticket
   iteration(0, IC<1>{});   // no P.V yet (and no V stage to read)
   for (int t = 1; t < n_tiles; ++t) iteration(t, IC<0>{});
