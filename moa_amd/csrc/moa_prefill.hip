@@ -167,9 +167,12 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
 
   // ---- the work queue ---------------------------------------------------------------------------
   // Thread 0 takes a ticket for the item after the one under way (from the own XCD's list while that has
-  // items, from the other lists then; never more than that one item in advance: items bound to a work-group
-  // early spread the items that run at the same time over more of a head's keys and cost L2 hits), turns it
-  // into an item descriptor once and leaves it in LDS; every wave reads it from there.
+  // items, from the other lists then), turns it into an item descriptor once and leaves it in LDS; every wave
+  // reads it from there.  The ticket is taken kTakeLead iterations before the item under way ends, not at its
+  // start: a ticket held through a long item starts late, behind tickets handed out after it, and the items
+  // of a head then run spread over the launch instead of side by side on their XCD (start order logged per
+  // item and replayed through an LRU model of the L2: 37 % of the K/V tile reads miss with tickets taken at
+  // the item's start, 22 % with late ones; measured HBM reads of the launch 2.2 GB against 1.2 GB).
   //   [0] n_tiles (-1: no more items)  [1] query tile  [2] ns  [3] nl  [4] lo2  [5] n_sink  [6] n_band  [7] band_rot
   //   [8,9] K base  [10,11] V base  [12,13] Q base (row 0 of the head)  [14,15] O base
   const int my_xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7;   // XCC_ID
@@ -202,23 +205,10 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
     if (list < 0) { d[0] = -1; return; }
     const int nb = (N + kKV - 1) / kKV;
     const bool sorted = Hkv <= kMaxSortedHeads;
-    // A list walks its pairs one after the other, late (long) query tiles first, and leaves the first
-    // n_last query tiles of every pair (causality keeps those short: query tile t sees at most 4 t + 4 key
-    // tiles) for the end, longest first across the pairs: heads differ little in span, so without them the
-    // last items handed out are as long as any and the CUs finish up to one whole item apart.
-    const int n_last = min(8, n_qtiles >> 2);
-    const int n_main = n_qtiles - n_last;
-    const int rounds = full_rounds + ((((full_rounds & 1) ? 7 - list : list) < rem) ? 1 : 0);
-    int round, qt;
-    if ((int)sq < rounds * n_main) {
-      const DivMod dm = divmod_small((int)sq, n_main);
-      round = dm.q;
-      qt = n_qtiles - 1 - dm.r;
-    } else {
-      const DivMod dm = divmod_small((int)sq - rounds * n_main, rounds);
-      qt = n_last - 1 - dm.q;
-      round = dm.r;
-    }
+    // A list walks its pairs one after the other, late (long) query tiles first.
+    const DivMod rq = divmod_small((int)sq, n_qtiles);
+    const int round = rq.q;
+    const int qt = n_qtiles - 1 - rq.r;
     const int pos = round * 8 + ((round & 1) ? 7 - list : list);   // position in the sorted list
     // sorted list: kv heads by rank; per kv head, batch-major, then the query heads of its group
     const DivMod ph = divmod_small(pos, per_head);   // (kv head rank, place inside the head's pairs)
@@ -431,9 +421,11 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
     continue;
   }
   if (!prefetched) start_copies(it, rst);
-  // the item after this one: thread 0 works its descriptor out while the loads above travel; every wave sees
-  // it after this item's first barrier
-  if (threadIdx.x == 0) take(par ^ 1);
+  // the item after this one: thread 0 works its descriptor out kTakeLead iterations before this item's last
+  // one (every wave sees it after the next barrier), or here when the item is that short
+  constexpr int kTakeLead = 6;
+  const int t_take = n_tiles - kTakeLead;
+  if (threadIdx.x == 0 && t_take < 1) take(par ^ 1);
 
   int jt[S];   // tiles of steps t .. t+S-1
   jt[0] = first_tile(it);
@@ -651,9 +643,14 @@ __global__ __launch_bounds__(512, 1) void prefill_kernel(PrefillArgs args_in_ker
 #pragma unroll
   for (int s = 0; s < KS; ++s) qf[s] ^= u32x4{q_sign, q_sign, q_sign, q_sign};
   asm volatile("" : "+v"(q_touch));   // the touch of the previous pass has landed as well
-  phase_barrier();               // K(0..2) and V(0..1) are in LDS; the next ticket is in s_ticket
+  phase_barrier();               // K(0..2) and V(0..1) are in LDS
   iteration(0, IC<1>{});   // no P.V yet (and no V stage to read)
-  for (int t = 1; t < n_tiles; ++t) iteration(t, IC<0>{});
+  {
+    int t = 1;
+    for (; t < t_take; ++t) iteration(t, IC<0>{});
+    if (threadIdx.x == 0 && t_take >= 1) take(par ^ 1);
+    for (; t < n_tiles; ++t) iteration(t, IC<0>{});
+  }
 
   // ---- iteration n_tiles: P.V of the last tile; the next item's first copies start here.
   // Every K stage is free by now (K(n_tiles-1) was read before the last barrier) and so are the V
