@@ -63,7 +63,7 @@ def parse_args():
                          "--new-tokens decode steps; not the contract line")
     ap.add_argument("--no-e2e", action="store_true",
                     help="skip the whole-decoder runs of the two end-to-end configurations in the default line")
-    ap.add_argument("--only", choices=["decode", "prefill", "copy", "e2e", "e2e-full", "gqa"], default=None,
+    ap.add_argument("--only", choices=["decode", "prefill", "copy", "e2e", "e2e-full", "gqa", "prompt"], default=None,
                     help="profiling aid: run one part only and print its figures (not the contract line)")
     return ap.parse_args()
 
@@ -749,6 +749,9 @@ def main():
         return
     if args.only == "gqa":
         print(json.dumps({"decode_gqa": bench_decode_gqa(torch, dev, args)}))
+        return
+    if args.only == "prompt":
+        print(json.dumps({"prompt_side": bench_prompt_side(torch, dev)}))
         return
     dec = bench_decode(torch, dev, args)
     rope = bench_rope_append(torch, dev, args, dec["cache"])

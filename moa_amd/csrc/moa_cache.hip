@@ -124,8 +124,10 @@ __device__ __forceinline__ HeadRing load_ring(const int64_t* update_index, const
 // With an attention mask: the positions of a batch row's valid tokens (mask == 1) in order,
 // tok_of[b, a] = position of the a-th valid token, and their number n_valid[b].  This is the inverse of
 // the reference's advancing_pos = cumsum(mask) - 1 (:1075-1080); its reversed_advancing_pos of a valid
-// token is n_valid - a (:1081-1086).  One work-group per batch row walks the row in slices of its size:
-// coalesced loads, a ballot and a population count inside each wave, the waves' totals through LDS.
+// token is n_valid - a (:1081-1086).  One work-group per batch row; every wave owns a contiguous segment
+// of the row and walks it twice with coalesced loads, a ballot and a population count per 64 tokens:
+// first to count its valid tokens (independent loads, nothing waits on LDS), then, once the waves'
+// totals have met in LDS (the only barrier), to write the positions from its offset on.
 constexpr int kScanThreads = 1024;
 __global__ __launch_bounds__(kScanThreads) void mask_compact_kernel(const int64_t* __restrict__ am,
                                                                      int64_t am_stride, int S,
@@ -137,26 +139,32 @@ __global__ __launch_bounds__(kScanThreads) void mask_compact_kernel(const int64_
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t* row = am + (int64_t)b * am_stride;
   int32_t* out = tok_of + (int64_t)b * S;
-  int base = 0;
-  for (int t0 = 0; t0 < S; t0 += kScanThreads) {
-    const int t = t0 + tid;
-    const bool valid = t < S && row[t] == 1;
-    const unsigned long long bal = __ballot(valid);
-    const int before = __popcll(bal & ((1ull << lane) - 1ull));
-    if (lane == 0) s_wave[wave] = __popcll(bal);
-    __syncthreads();
-    int off = 0, total = 0;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      const int c = s_wave[w];
-      off += (w < wave) ? c : 0;
-      total += c;
-    }
-    if (valid) out[base + off + before] = t;
-    base += total;
-    __syncthreads();   // s_wave is written again in the next slice
+  const int seg = ((S + kWaves - 1) / kWaves + 63) & ~63;   // tokens per wave, a multiple of 64
+  const int t_begin = min(S, wave * seg), t_end = min(S, t_begin + seg);
+  int mine = 0;
+#pragma unroll 4
+  for (int t0 = t_begin; t0 < t_end; t0 += 64) {
+    const int t = t0 + lane;
+    mine += __popcll(__ballot(t < t_end && row[t] == 1));
   }
-  if (tid == 0) n_valid[b] = base;
+  if (lane == 0) s_wave[wave] = mine;
+  __syncthreads();
+  int base = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) {
+    const int c = s_wave[w];
+    base += (w < wave) ? c : 0;
+    total += c;
+  }
+#pragma unroll 4
+  for (int t0 = t_begin; t0 < t_end; t0 += 64) {
+    const int t = t0 + lane;
+    const bool valid = t < t_end && row[t] == 1;
+    const unsigned long long bal = __ballot(valid);
+    if (valid) out[base + __popcll(bal & ((1ull << lane) - 1ull))] = t;
+    base += __popcll(bal);
+  }
+  if (tid == 0) n_valid[b] = total;
 }
 
 constexpr int kRowsPerThread = 4;   // rows a group of 16 lanes moves: all loads go out before the first store
@@ -210,32 +218,27 @@ __global__ __launch_bounds__(kCacheThreads) void cache_prefill_copy_kernel(
   }
 }
 
-// One wavefront per (b, h): count the kept tokens, then move the pointers
-// (:1110, :1136-1138).  Runs after the copy kernel on the same stream because
-// it overwrites update_index, which the copy kernel reads.
+// One thread per (b, h): add the number of kept tokens to the valid length, then move the pointer
+// (:1110, :1136-1138).  Runs after the copy kernel on the same stream because it overwrites
+// update_index, which the copy kernel reads.  The count has a closed form in the candidates' terms:
+// the last min(csz, n_valid) valid tokens have rap <= csz and are all kept; of the earlier ones
+// (a < n_valid - csz, so rap > csz) exactly those are kept whose slot lies in front of the ring, which
+// needs a non-circular slot (kv0 + a <= s, then slot = upd0 + a) below the ring's first row.
 __global__ __launch_bounds__(256) void cache_prefill_index_kernel(
     int64_t* __restrict__ update_index, int64_t* __restrict__ valid_len,
     const int64_t* __restrict__ circ_head, const int64_t* __restrict__ circ_size,
     const int64_t* __restrict__ static_size, const int32_t* __restrict__ n_valid, int64_t kv_len, int B, int H,
     int S) {
-  const int lane = threadIdx.x & 63;
-  const int64_t bh = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t bh = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (bh >= (int64_t)B * H) return;
   const int b = (int)(bh / H);
   const int h = (int)(bh % H);
   const HeadRing g = load_ring(update_index, circ_head, circ_size, static_size, kv_len, bh, h);
   const int64_t nv = n_valid ? (int64_t)n_valid[b] : (int64_t)S;
-  const int64_t n_cand = candidate_count(g, nv);
-  int count = 0;
-  for (int64_t r = lane; r < n_cand; r += 64) {
-    int64_t a, slot;
-    count += candidate(g, r, nv, a, slot) ? 1 : 0;
-  }
-  for (int off = 32; off > 0; off >>= 1) count += __shfl_xor(count, off, 64);
-  if (lane == 0) {
-    update_index[bh] = slot_of(g, nv);   // the slot the token after the last valid one would take (:1110)
-    valid_len[bh] += count;
-  }
+  const int64_t recent = min(g.csz, nv);
+  const int64_t early = max((int64_t)0, min(min(nv - g.csz, g.s + 1), min(g.s - g.kv0 + 1, g.ch - g.upd0)));
+  update_index[bh] = slot_of(g, nv);   // the slot the token after the last valid one would take (:1110)
+  valid_len[bh] += recent + early;
 }
 
 static int check_rows(const char* who, int D, int dtype, const int64_t* strides, int nstr,
@@ -353,7 +356,7 @@ extern "C" int moa_cache_prefill_insert(const void* k, const void* v, const int6
     if (rc) return rc;
   }
   const int64_t n = (int64_t)B * H;
-  hipLaunchKernelGGL(cache_prefill_index_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, st,
+  hipLaunchKernelGGL(cache_prefill_index_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
                      update_index, valid_len, circ_head, circ_size, static_size, (const int32_t*)n_valid, kv_len, B, H,
                      S);
   return check_launch("moa_cache_prefill_insert(index)");
