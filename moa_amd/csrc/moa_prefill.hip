@@ -18,9 +18,9 @@
 //     work-group per item a CU that falls free waits until it is its XCD's turn
 //     (measured: 7 % of CU time at the benchmark shape);
 //   * thread 0 turns a queue ticket into an item descriptor (base pointers, tile
-//     schedule) once and leaves it in LDS; it does so for item i+1 while the
-//     loads of item i travel, and item i's last iteration starts the first
-//     copies of item i+1;
+//     schedule) once and leaves it in LDS; it does so for item i+1 a few
+//     iterations before item i ends, and item i's last iteration starts the
+//     first copies of item i+1;
 //   * a work-group walks the union of the live 64-key tiles of its four query
 //     blocks; a wave skips the math of a tile that is dead for ITS query block;
 //   * K and V tiles are copied global -> LDS asynchronously (no registers),
