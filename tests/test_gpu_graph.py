@@ -79,3 +79,74 @@ def test_decode_step_replays_like_eager(dev, G):
         assert torch.equal(cache_g.value_cache[0], cache_e.value_cache[0]), t
         assert torch.equal(cache_g.cache_update_index[0], cache_e.cache_update_index[0]), t
         assert torch.equal(cache_g.cache_valid_length[0], cache_e.cache_valid_length[0]), t
+
+
+def test_prompt_pass_replays_like_eager(dev):
+    """The prompt side recorded into a HIP graph: rotary embedding, block-sparse prefill (its work queue is
+    a slot of a device array chosen at record time: every replay of the graph reuses that slot, one after
+    the other on a stream), bulk insert into the rings.  One ordinary call comes first, as the header asks
+    (the first call on a device looks up device addresses, which a capture cannot contain).  Every replay
+    runs on new inputs and must equal the same calls run eagerly, bit for bit, rings and indices included."""
+    import copy
+
+    from moa_amd import StaticCircularCache, mixture_of_sparse_attention
+    from moa_amd.kernels.rotary import apply_rotary_pos_emb
+    B, Hq, Hkv, N, D = 2, 8, 4, 1000, 128
+    dtype = torch.bfloat16
+    sink = torch.tensor([64, 64, 128, 0], device=dev)
+    local = torch.tensor([128, 512, 256, 1024], device=dev)
+    cache_size = [int(s + l) for s, l in zip(sink.tolist(), local.tolist())]
+    cos, sin = rope_cos_sin(torch.arange(N)[None, :].expand(B, N), D, dtype=dtype)
+    cos, sin = cos.to(dev), sin.to(dev)
+
+    def fresh_cache():
+        return StaticCircularCache([cache_size], static_size=[sink.tolist()], batch_size=B, head_dim=D, device=dev,
+                                   dtype=dtype)
+
+    def prompt(cache, q, k, v):
+        qe, ke = apply_rotary_pos_emb(q, k, cos, sin)
+        out = mixture_of_sparse_attention(qe, ke, v, D ** -0.5, sink_size=sink, local_size=local)
+        cache.update(ke, v, 0)
+        return out
+
+    g = torch.Generator().manual_seed(5)
+    def draw():
+        q = torch.randn(B, N, Hq, D, generator=g).to(dev, dtype).transpose(1, 2)
+        k, v = (torch.randn(B, N, Hkv, D, generator=g).to(dev, dtype).transpose(1, 2) for _ in range(2))
+        return q, k, v
+
+    q0, k0, v0 = draw()
+    prompt(fresh_cache(), q0, k0, v0)            # set-up calls outside any capture
+    torch.cuda.synchronize()
+
+    sq, sk, sv = (t.clone() for t in (q0, k0, v0))   # static inputs of the graph
+    cache_g = fresh_cache()
+    cache_g._to_device(0, dev)                       # rings and index arrays allocated before the state is saved
+    pristine = copy.deepcopy(cache_g)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        prompt(copy.deepcopy(pristine), sq, sk, sv)  # allocator warm-up on the capture stream
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            out_g = prompt(cache_g, sq, sk, sv)
+    torch.cuda.current_stream().wait_stream(stream)
+
+    index_names = ("cache_update_index", "cache_valid_length", "mask_cache")
+    for rep in range(3):
+        q, k, v = draw()
+        # the rings and indices go back to their state at record time, with fill kernels (copy_)
+        cache_g.key_cache[0].copy_(pristine.key_cache[0]); cache_g.value_cache[0].copy_(pristine.value_cache[0])
+        for name in index_names:
+            getattr(cache_g, name)[0].copy_(getattr(pristine, name)[0])
+        sq.copy_(q); sk.copy_(k); sv.copy_(v)
+        graph.replay()
+        torch.cuda.synchronize()
+        cache_e = copy.deepcopy(pristine)
+        out_e = prompt(cache_e, q, k, v)
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, out_e), rep
+        assert torch.equal(cache_g.key_cache[0], cache_e.key_cache[0]) and torch.equal(cache_g.value_cache[0], cache_e.value_cache[0]), rep
+        for name in index_names:
+            assert torch.equal(getattr(cache_g, name)[0], getattr(cache_e, name)[0]), (rep, name)
