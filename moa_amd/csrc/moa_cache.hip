@@ -125,9 +125,10 @@ __device__ __forceinline__ HeadRing load_ring(const int64_t* update_index, const
 // tok_of[b, a] = position of the a-th valid token, and their number n_valid[b].  This is the inverse of
 // the reference's advancing_pos = cumsum(mask) - 1 (:1075-1080); its reversed_advancing_pos of a valid
 // token is n_valid - a (:1081-1086).  One work-group per batch row; every wave owns a contiguous segment
-// of the row and walks it twice with coalesced loads, a ballot and a population count per 64 tokens:
-// first to count its valid tokens (independent loads, nothing waits on LDS), then, once the waves'
-// totals have met in LDS (the only barrier), to write the positions from its offset on.
+// of the row and walks it twice, a lane looking at four consecutive tokens per step: first to count its
+// valid tokens (independent loads, nothing waits on LDS), then, once the waves' totals have met in LDS
+// (the only barrier), to write the positions from its offset on (ballots and population counts give a
+// lane the number of valid tokens in front of its four).
 constexpr int kScanThreads = 1024;
 __global__ __launch_bounds__(kScanThreads) void mask_compact_kernel(const int64_t* __restrict__ am,
                                                                      int64_t am_stride, int S,
@@ -139,14 +140,19 @@ __global__ __launch_bounds__(kScanThreads) void mask_compact_kernel(const int64_
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t* row = am + (int64_t)b * am_stride;
   int32_t* out = tok_of + (int64_t)b * S;
-  const int seg = ((S + kWaves - 1) / kWaves + 63) & ~63;   // tokens per wave, a multiple of 64
+  constexpr int kPerLane = 4;              // consecutive tokens a lane looks at per step
+  constexpr int kStep = 64 * kPerLane;
+  const int seg = ((S + kWaves - 1) / kWaves + kStep - 1) / kStep * kStep;   // tokens per wave, whole steps
   const int t_begin = min(S, wave * seg), t_end = min(S, t_begin + seg);
   int mine = 0;
 #pragma unroll 4
-  for (int t0 = t_begin; t0 < t_end; t0 += 64) {
-    const int t = t0 + lane;
-    mine += __popcll(__ballot(t < t_end && row[t] == 1));
+  for (int t0 = t_begin; t0 < t_end; t0 += kStep) {
+    const int t = t0 + kPerLane * lane;
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j) mine += (t + j < t_end && row[t + j] == 1) ? 1 : 0;
   }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mine += __shfl_xor(mine, off, 64);
   if (lane == 0) s_wave[wave] = mine;
   __syncthreads();
   int base = 0, total = 0;
@@ -156,13 +162,26 @@ __global__ __launch_bounds__(kScanThreads) void mask_compact_kernel(const int64_
     base += (w < wave) ? c : 0;
     total += c;
   }
+  const unsigned long long below = (1ull << lane) - 1ull;
 #pragma unroll 4
-  for (int t0 = t_begin; t0 < t_end; t0 += 64) {
-    const int t = t0 + lane;
-    const bool valid = t < t_end && row[t] == 1;
-    const unsigned long long bal = __ballot(valid);
-    if (valid) out[base + __popcll(bal & ((1ull << lane) - 1ull))] = t;
-    base += __popcll(bal);
+  for (int t0 = t_begin; t0 < t_end; t0 += kStep) {
+    const int t = t0 + kPerLane * lane;
+    bool valid[kPerLane];
+    int before = 0, step_total = 0;   // valid tokens of lower lanes; of the whole step
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j) {
+      valid[j] = t + j < t_end && row[t + j] == 1;
+      const unsigned long long bal = __ballot(valid[j]);
+      before += __popcll(bal & below);
+      step_total += __popcll(bal);
+    }
+    int at = base + before;
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j) {
+      if (valid[j]) out[at] = t + j;
+      at += valid[j] ? 1 : 0;
+    }
+    base += step_total;
   }
   if (tid == 0) n_valid[b] = total;
 }
