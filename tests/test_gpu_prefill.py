@@ -186,6 +186,30 @@ def test_many_heads_with_equal_and_extreme_spans(dev):
     assert torch.equal(out2.transpose(1, 2), out)
 
 
+def test_many_launches_in_flight_on_two_streams(dev):
+    """The work queue of a launch is one of 256 slots of a device array, handed out in turn and cleared by
+    the launch's last work-group.  600 launches of two different shapes, alternating between two streams
+    with nothing waiting in between (so launches overlap and the slots go round more than twice): every
+    result must equal that of the same call made alone, bit for bit."""
+    shapes = [(2, 6, 700, 64, torch.float16, [1, 0, 2, 1, 1, 3], [2, 5, 1, 11, 3, 4]),
+              (1, 4, 1300, 128, torch.bfloat16, [1, 1, 0, 2], [4, 21, 2, 7])]
+    cases = []
+    for i, (B, H, N, D, dtype, ns, nl) in enumerate(shapes):
+        q, k, v = _qkv(B, H, N, D, dtype, dev, seed=70 + i)
+        alone = _run(q, k, v, D ** -0.5, ns, nl, dev).clone()
+        cases.append((q, k, v, D ** -0.5, ns, nl, alone))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = []
+    for i in range(600):
+        q, k, v, sm, ns, nl, alone = cases[i % 2]
+        with torch.cuda.stream(streams[(i // 2) % 2]):
+            outs.append((i % 2, _run(q, k, v, sm, ns, nl, dev)))
+    torch.cuda.synchronize()
+    for i, (c, out) in enumerate(outs):
+        assert torch.equal(out, cases[c][6]), i
+
+
 def test_gqa_70b_shape(dev):
     """The largest config's head layout: 64 query heads on 8 kv heads, head_dim 128, bf16 (its
     32k-token prompt shortened to 4096 so that the CPU oracle finishes in seconds)."""
