@@ -163,7 +163,6 @@ __global__ __launch_bounds__(kScanThreads) void mask_compact_kernel(const int64_
     total += c;
   }
   const unsigned long long below = (1ull << lane) - 1ull;
-#pragma unroll 4
   for (int t0 = t_begin; t0 < t_end; t0 += kStep) {
     const int t = t0 + kPerLane * lane;
     bool valid[kPerLane];
