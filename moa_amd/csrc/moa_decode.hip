@@ -107,6 +107,7 @@ struct HeadTable {
   int prefix[kMaxHeads + 1];
   int seg0[kMaxHeads];   // first cache row of the head's segment (rows per batch row fit 31 bits: checked on the host)
   int len[kMaxHeads];    // valid rows, clamped to the end of the batch row
+  int clen[kMaxHeads];   // rows per chunk of this head
 };
 
 template <int CHUNK, int NWAVES = kDecWaves>
@@ -123,6 +124,7 @@ __device__ __forceinline__ int build_prefix(const int64_t* __restrict__ valid_ro
     if (len > sumC - seg0) len = sumC - seg0;
     tab->seg0[tid] = (int)(len > 0 ? seg0 : 0);
     tab->len[tid] = (int)len;
+    tab->clen[tid] = CHUNK;
     n = (int)((len + CHUNK - 1) / CHUNK);
   }
   int incl = n;   // inclusive scan inside the wave
@@ -150,6 +152,80 @@ __device__ __forceinline__ int find_head(const int* __restrict__ s_prefix, int H
     if (s_prefix[mid] <= w) lo = mid; else hi = mid;
   }
   return lo;
+}
+
+// The same table with chunks of about equal length over the whole batch row instead of a fixed chunk
+// length.  With a fixed length the last chunk of every head is a remainder and the number of chunks is
+// whatever it comes to; here the caller names the number of chunks (`target`) a batch row should not
+// exceed, and the table takes the shortest chunk length c (whole steps of kEvenStep rows, at least
+// kEvenMinChunk) for which sum_h ceil(len_h / c) <= target; head h is then split evenly into
+// ceil(len_h / c) chunks.  The search starts at total / target and goes up step by step (the sum exceeds
+// the target by at most the number of heads at the start, so a few steps do), and gives up after
+// kEvenTries: the table is valid for any c, the target is a wish.  Integer arithmetic only: the split
+// and the merge kernel build this table independently and must agree on every entry.
+constexpr int kEvenMinChunk = 256;   // also the chunk length the partial slots of a batch row are sized for
+constexpr int kEvenStep = 128;
+constexpr int kEvenTries = 24;
+template <int NWAVES>
+__device__ __forceinline__ int build_prefix_even(const int64_t* __restrict__ valid_row, const int64_t* __restrict__ start_row,
+                                                 int H, int64_t sumC, int cap, int target, HeadTable* __restrict__ tab) {
+  __shared__ int s_wave_total[NWAVES];
+  __shared__ int s_wave_sum[2][NWAVES];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  int len = 0;
+  if (tid < H) {
+    int64_t l = valid_row[tid];
+    const int64_t seg0 = start_row[tid];
+    if (l < 0 || seg0 < 0 || seg0 >= sumC) l = 0;
+    if (l > sumC - seg0) l = sumC - seg0;
+    tab->seg0[tid] = (int)(l > 0 ? seg0 : 0);
+    tab->len[tid] = (int)l;
+    len = (int)l;
+  }
+  // sum over the work-group of a per-thread count (every thread gets the sum); `buf` alternates so that
+  // one barrier per call is enough
+  auto block_sum = [&](int x, int buf) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off, 64);
+    if (lane == 0) s_wave_sum[buf][wave] = x;
+    __syncthreads();
+    int t = 0;
+#pragma unroll
+    for (int w = 0; w < NWAVES; ++w) t += s_wave_sum[buf][w];
+    return t;
+  };
+  // rows of the batch row in steps (a sum of at most 256 heads of < 2^31 rows each fits 32 bits in steps)
+  const int total_steps = block_sum((len + kEvenStep - 1) / kEvenStep, 0);
+  int c = max(kEvenMinChunk, ((total_steps + target - 1) / max(target, 1)) * kEvenStep);
+  int n = 0;
+  for (int i = 0; i < kEvenTries; ++i) {
+    n = (len + c - 1) / c;
+    if (block_sum(n, (i + 1) & 1) <= target) break;   // the same for every thread
+    c += kEvenStep;
+    n = (len + c - 1) / c;   // what the table holds if this was the last try
+  }
+  int clen = kEvenStep;
+  if (n > 0) {
+    clen = (((len + n - 1) / n + kEvenStep - 1) / kEvenStep) * kEvenStep;   // even split, <= c
+    n = (len + clen - 1) / clen;
+  }
+  if (tid < kMaxHeads) tab->clen[tid] = clen;
+  int incl = n;   // inclusive scan inside the wave
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int up = __shfl_up(incl, off, 64);
+    if (lane >= off) incl += up;
+  }
+  if (lane == 63) s_wave_total[wave] = incl;
+  __syncthreads();
+  int base = 0;
+#pragma unroll
+  for (int w = 0; w < NWAVES; ++w) base += (w < wave) ? s_wave_total[w] : 0;
+  if (tid < kMaxHeads) tab->prefix[tid + 1] = min(base + incl, cap);
+  if (tid == 0) tab->prefix[0] = 0;
+  __syncthreads();
+  return tab->prefix[H];
 }
 
 // H: kv heads (rings) per batch row; query head hk*G + g reads ring hk.
@@ -357,7 +433,8 @@ template <typename T, int D, int CHUNK>
 __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
     uint16_t* __restrict__ o, const float* __restrict__ part_acc, const float* __restrict__ part_ml,
     const int64_t* __restrict__ head_start, const int64_t* __restrict__ head_valid, int H,
-    int G /* query heads per ring */, int64_t sumC, int cap) {
+    int G /* query heads per ring */, int64_t sumC, int cap,
+    int even_target /* > 0: the split kernel used build_prefix_even with this target */) {
   constexpr int GROUPS = kDecThreads / D;
   constexpr int kFactors = 64;   // chunks whose factors are staged at a time
   __shared__ HeadTable s_tab;
@@ -366,7 +443,10 @@ __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
   __shared__ int s_n[GROUPS];
   const int b = blockIdx.y;
   const int tid = threadIdx.x;
-  build_prefix<CHUNK>(head_valid + (int64_t)b * H, head_start + (int64_t)b * H, H, sumC, cap, &s_tab);
+  if (even_target > 0)
+    build_prefix_even<kDecWaves>(head_valid + (int64_t)b * H, head_start + (int64_t)b * H, H, sumC, cap, even_target, &s_tab);
+  else
+    build_prefix<CHUNK>(head_valid + (int64_t)b * H, head_start + (int64_t)b * H, H, sumC, cap, &s_tab);
   const int grp = tid / D;
   const int d = tid % D;
   // every group runs the same number of rounds so that the barriers below are uniform
@@ -451,9 +531,10 @@ __global__ __launch_bounds__(kDecThreads) void decode_merge_kernel(
 // dispatcher hands out chunks as CUs become free when every chunk is a work-group of its own: 602 us at
 // batch 64 of the 70B shape against 612-628 us with 2-16 per CU, each walking several chunks in a fixed order.
 constexpr int kGqaBlocksPerCu = 64;
-// Cache rows per work-group step (a quarter per wave).  A chunk start costs a wave full memory
-// latencies with nothing in flight, so long chunks win: 2048 is the best of 512..4096 at batch 64 and at
-// batch 4.
+// Largest number of cache rows per work-group step (a quarter per wave) the launch aims for; the actual
+// chunk lengths come out of an even split of every batch row (build_prefix_even).  A chunk start costs a
+// wave full memory latencies with nothing in flight, so long chunks win: with one fixed length, 2048 was
+// the best of 512..4096 at batch 64 and at batch 4.
 constexpr int kGqaChunk = 2048;
 constexpr int kGqaTile = 32;      // keys per MFMA tile
 constexpr int kGqaMaxG = 8;       // query heads per ring the per-wave result buffers are sized for
@@ -468,12 +549,13 @@ template <> struct MfmaElem<BF16> { typedef PBF16 type; };
 template <int D>
 constexpr size_t gqa_lds_bytes() { return (size_t)kGqaWaves * kGqaStages * 2 * kGqaTile * D * 2; }
 
-template <typename T, int D, int CHUNK>
+template <typename T, int D>
 __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
     uint16_t* __restrict__ o, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const int64_t* __restrict__ head_start, const int64_t* __restrict__ head_valid, int H,
-    int G /* query heads per ring, <= kGqaMaxG */, int64_t sumC, float scale_log2_signed, int cap) {
+    int G /* query heads per ring, <= kGqaMaxG */, int64_t sumC, float scale_log2_signed, int cap,
+    int target /* > 0: chunks a batch row is split into (build_prefix_even); 0: chunks of kGqaChunk rows */) {
   typedef typename MfmaElem<T>::type M;
   // the row maximum is taken over unscaled scores: a negative softmax scale goes into Q (sign flip, exact)
   const float scale_log2 = __builtin_fabsf(scale_log2_signed);
@@ -486,9 +568,8 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
   constexpr int TILE_B = kGqaTile * ROW_B;      // bytes of one K or V tile
   constexpr int NCP = TILE_B / 1024;            // async copies per tile and tensor
   constexpr int STAGE_B = 2 * TILE_B;           // K tile, then V tile
-  constexpr int WCHUNK = CHUNK / kGqaWaves;
   constexpr float kRescaleStep = 8.f;
-  static_assert(WCHUNK % kGqaTile == 0, "a wave's share of a chunk is whole tiles");
+  static_assert((kEvenStep / kGqaWaves) % kGqaTile == 0, "a wave's share of a chunk is whole tiles");
 
   extern __shared__ __attribute__((aligned(1024))) char s_mem[];
   __shared__ HeadTable s_tab;
@@ -532,7 +613,9 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
     for (int dt = 0; dt < DT; ++dt) v_ad[dt] = ring0 + TILE_B + (v_rd ^ (uint32_t)(64 * dt));
   }
 
-  const int total = build_prefix<CHUNK, kGqaWaves>(head_valid + (int64_t)b * H, head_start + (int64_t)b * H, H, sumC, cap, &s_tab);
+  const int total = target > 0
+      ? build_prefix_even<kGqaWaves>(head_valid + (int64_t)b * H, head_start + (int64_t)b * H, H, sumC, cap, target, &s_tab)
+      : build_prefix<kGqaChunk, kGqaWaves>(head_valid + (int64_t)b * H, head_start + (int64_t)b * H, H, sumC, cap, &s_tab);
 
   for (int w = blockIdx.x; w < total; w += gridDim.x) {
     const int h = find_head(s_prefix, H, w);
@@ -541,8 +624,10 @@ __global__ __launch_bounds__(kGqaThreads) void decode_gqa_kernel(
     const int64_t bh = (int64_t)b * H + h;
     const int64_t seg0 = s_tab.seg0[h];
     const int64_t len = s_tab.len[h];
-    const int64_t r_begin = (int64_t)c * CHUNK + (int64_t)wave * WCHUNK;
-    int64_t r_end = r_begin + WCHUNK;
+    const int clen = s_tab.clen[h];            // rows of one chunk of this head
+    const int wchunk = clen / kGqaWaves;       // a wave's share: whole tiles
+    const int64_t r_begin = (int64_t)c * clen + (int64_t)wave * wchunk;
+    int64_t r_end = r_begin + wchunk;
     if (r_end > len) r_end = len;
     const int n_rows = __builtin_amdgcn_readfirstlane(r_end > r_begin ? (int)(r_end - r_begin) : 0);
     const int n_t = (n_rows + kGqaTile - 1) / kGqaTile;
@@ -741,7 +826,7 @@ static int launch_decode(const void* q, const void* kc, const void* vc, void* o,
     int rc = check_launch("moa_decode_fwd(split)");
     if (rc) return rc;
     hipLaunchKernelGGL((decode_merge_kernel<T, D, kSmallChunk>), dim3(mx, B), dim3(kDecThreads), 0, st,
-                       (uint16_t*)o, part_acc, part_ml, head_start, head_valid, H, G, sumC, cap);
+                       (uint16_t*)o, part_acc, part_ml, head_start, head_valid, H, G, sumC, cap, 0);
     return check_launch("moa_decode_fwd(merge)");
   }
   if (pipe)
@@ -755,46 +840,53 @@ static int launch_decode(const void* q, const void* kc, const void* vc, void* o,
   int rc = check_launch("moa_decode_fwd(split)");
   if (rc) return rc;
   hipLaunchKernelGGL((decode_merge_kernel<T, D, kChunk>), dim3(mx, B), dim3(kDecThreads), 0, st,
-                     (uint16_t*)o, part_acc, part_ml, head_start, head_valid, H, G, sumC, cap);
+                     (uint16_t*)o, part_acc, part_ml, head_start, head_valid, H, G, sumC, cap, 0);
   return check_launch("moa_decode_fwd(merge)");
 }
 
-
-template <typename T, int D, int CHUNK>
-static int launch_decode_gqa_chunk(const void* q, const void* kc, const void* vc, void* o, float* part_acc,
-                                   float* part_ml, const int64_t* head_start, const int64_t* head_valid, int B,
-                                   int H, int G, int64_t sumC, float sm_scale, hipStream_t st) {
-  const int cap = (int)decode_cap(sumC, H);   // partial slots per batch row the workspace was sized for
-  const int64_t chunks = (sumC + CHUNK - 1) / CHUNK + H;   // at most this many steps per batch row
-  int bx = (int)((256 * kGqaBlocksPerCu + B - 1) / B);   // in practice one work-group per chunk (see kGqaBlocksPerCu)
-  if (bx > chunks) bx = (int)chunks;
-  if (bx < 1) bx = 1;
-  constexpr size_t lds = gqa_lds_bytes<D>();
-  static bool lds_reserved[kMaxDevices] = {};   // per template instance
-  if (int rc = reserve_lds(reinterpret_cast<const void*>(&decode_gqa_kernel<T, D, CHUNK>), lds, lds_reserved, "moa_decode_fwd"))
-    return rc;
-  hipLaunchKernelGGL((decode_gqa_kernel<T, D, CHUNK>), dim3(bx, B), dim3(kGqaThreads), lds, st,
-                     (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, (uint16_t*)o,
-                     part_acc, part_ml, head_start, head_valid, H, G, sumC, mfma_softmax_scale(sm_scale), cap);
-  int rc = check_launch("moa_decode_fwd(grouped split)");
-  if (rc) return rc;
-  constexpr int GROUPS = kDecThreads / D;
-  int mx = (H * G + GROUPS - 1) / GROUPS;
-  hipLaunchKernelGGL((decode_merge_kernel<T, D, CHUNK>), dim3(mx, B), dim3(kDecThreads), 0, st,
-                     (uint16_t*)o, part_acc, part_ml, head_start, head_valid, H, G, sumC, cap);
-  return check_launch("moa_decode_fwd(merge)");
-}
 
 template <typename T, int D>
 static int launch_decode_gqa(const void* q, const void* kc, const void* vc, void* o, float* part_acc,
                              float* part_ml, const int64_t* head_start, const int64_t* head_valid, int B,
                              int H, int G, int64_t sumC, float sm_scale, hipStream_t st) {
-  // One chunk length for every launch.  Measured at batch 4 of the 70B shape (213 MB of rings, about one
-  // 2048-row chunk per CU): 49.8 us per call with 2048-row chunks, 53.3 with 1024, 62.3 with 512 -- a chunk
-  // start costs three dependent memory latencies (ring index, query rows, first tiles), which shorter
-  // chunks pay more often than they win in balance.
-  return launch_decode_gqa_chunk<T, D, kGqaChunk>(q, kc, vc, o, part_acc, part_ml, head_start, head_valid, B, H, G, sumC,
-                                                  sm_scale, st);
+  const int cap = (int)decode_cap(sumC, H);   // partial slots per batch row the workspace was sized for
+  // Chunk policy.  Chunks of kGqaChunk rows when they give at least half of the CUs a chunk: measured at
+  // the 70B shape (8 rings per batch row, 104 k rows) with one fixed length, 49.8 us per call at batch 4
+  // with 2048-row chunks, 53.3 with 1024, 62.3 with 512 -- a chunk start costs three dependent memory
+  // latencies (ring index, query rows, first tiles).  Below that (batch 1 and 2 at that shape: 54 and 108
+  // chunks) every batch row is split evenly into its share of 256 chunks instead: 25.8 against 32.4 us at
+  // batch 1, 33.5 against 36-39 us at batch 2.  From batch 3 on the even split gains nothing (one round of
+  // 256 chunks of 1664 rows at batch 4: 50.6-52.2 us against 50.4-51.8 us with 213 chunks of 2048; whole
+  // rounds of even chunks at batch 6 to 64: between 4 % faster and 7 % slower): those launches stream at
+  // the rate of the large batches already.  The host does not know how full the rings are; it plans with
+  // their capacity.
+  const int64_t fixed_chunks = (int64_t)B * (sumC / kGqaChunk + (H + 1) / 2);
+  int64_t target = 0;   // 0: chunks of kGqaChunk rows
+  if (fixed_chunks <= 128) {
+    target = (256 + B - 1) / B;
+    if (target > cap) target = cap;
+  }
+  // at most this many chunks per batch row (a work-group without a chunk still holds a CU while it finds that out)
+  const int64_t chunks = target > 0 ? target + H : (sumC + kGqaChunk - 1) / kGqaChunk + H;
+  int64_t bx = (256 * kGqaBlocksPerCu + B - 1) / B;   // in practice one work-group per chunk (see kGqaBlocksPerCu)
+  if (bx > chunks) bx = chunks;
+  if (bx > cap) bx = cap;
+  if (bx < 1) bx = 1;
+  constexpr size_t lds = gqa_lds_bytes<D>();
+  static bool lds_reserved[kMaxDevices] = {};   // per template instance
+  if (int rc = reserve_lds(reinterpret_cast<const void*>(&decode_gqa_kernel<T, D>), lds, lds_reserved, "moa_decode_fwd"))
+    return rc;
+  hipLaunchKernelGGL((decode_gqa_kernel<T, D>), dim3((unsigned)bx, B), dim3(kGqaThreads), lds, st,
+                     (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, (uint16_t*)o,
+                     part_acc, part_ml, head_start, head_valid, H, G, sumC, mfma_softmax_scale(sm_scale), cap,
+                     (int)target);
+  int rc = check_launch("moa_decode_fwd(grouped split)");
+  if (rc) return rc;
+  constexpr int GROUPS = kDecThreads / D;
+  int mx = (H * G + GROUPS - 1) / GROUPS;
+  hipLaunchKernelGGL((decode_merge_kernel<T, D, kGqaChunk>), dim3(mx, B), dim3(kDecThreads), 0, st,
+                     (uint16_t*)o, part_acc, part_ml, head_start, head_valid, H, G, sumC, cap, (int)target);
+  return check_launch("moa_decode_fwd(merge)");
 }
 
 // Launches the decode kernels with their partials in `workspace` (at least

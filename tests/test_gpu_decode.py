@@ -281,6 +281,31 @@ def test_grouped_query_boundaries_and_invariants(dev, G, B):
     assert (ones.float() - expect.float()).abs().max().item() <= 1e-3
 
 
+@pytest.mark.parametrize("B", [1, 2])
+def test_grouped_query_small_batch_even_split(dev, B):
+    """Batch 1 and 2 at the largest config's ring sizes (8 rings of 2 k to 24 k rows, 8 query heads each,
+    bf16): too few 2048-row chunks for the chip, so the kernel splits every batch row evenly into its share
+    of 256 chunks, with a chunk length per ring found on the device from the valid lengths.  The batch rows
+    are filled differently (full; partly, with one empty ring and one of a single row), so each has its own
+    table; whole output against the oracle."""
+    from moa_amd import mixture_of_sparse_attention
+    from moa_amd.workloads import elastic_spans, ring_cache_sizes
+    rng = np.random.default_rng(300 + B)
+    G, D, dtype = 8, 128, torch.bfloat16
+    sizes = ring_cache_sizes(elastic_spans(8, 32768, seed=3, alpha_range=(256.0, 8192.0)))[0]
+    Hkv = len(sizes)
+    _, kc, vc, hs, hv = _case(rng, B, sizes, D, dtype, dev)
+    if B > 1:
+        hv[1] = np.maximum(1, (hv[1] * rng.uniform(0.05, 0.9, size=Hkv)).astype(np.int64))
+        hv[1, 2], hv[1, 5] = 0, 1
+    q = torch.from_numpy(rng.standard_normal((B, Hkv * G, 1, D)).astype(np.float32)).to(dev, dtype)
+    out = mixture_of_sparse_attention(q, kc, vc, D ** -0.5, head_start_index=torch.from_numpy(hs).to(dev),
+                                      head_valid_length=torch.from_numpy(hv).to(dev))
+    _close_grouped(out[:, 0], q[:, :, 0], kc, vc, hs, hv, D ** -0.5, G, ("gqa even split", B))
+    if B > 1:
+        assert not out[1, 0, 2 * G:3 * G].any()
+
+
 @pytest.mark.parametrize("seed", range(16))
 def test_random_layouts(dev, seed):
     """Segments anywhere in the packed row (gaps between them, not in head order), random valid
