@@ -762,10 +762,13 @@ static int launch_prefill(const void* q, const void* k, const void* v, void* o, 
   constexpr int NW = 8, S = 4;
   constexpr int kQRows = NW * kWRows;
   const int n_qtiles = (N + kQRows - 1) / kQRows;
-  const int BH = B * Hq;
-  const int64_t items = (int64_t)BH * n_qtiles;
-  // the queue's ticket arithmetic (divmod_small) is exact below 2^22 per list of an XCD
-  if (items > (1LL << 25) || N > (1 << 28)) return fail(MOA_ERR_UNSUPPORTED, "moa_prefill_fwd: too many work items");
+  const int64_t pairs = (int64_t)B * Hq;
+  const int64_t items = pairs * n_qtiles;
+  // the queue's ticket arithmetic (divmod_small) is exact below 2^22: tickets of one XCD's list (an eighth
+  // of the items) and positions in the list of (batch, head) pairs
+  if (items > (1LL << 25) || pairs > (1LL << 22) || N > (1 << 28))
+    return fail(MOA_ERR_UNSUPPORTED, "moa_prefill_fwd: too many work items");
+  const int BH = (int)pairs;
   // the async copies address a tile row through a 32-bit element offset
   if (64 * ks[2] + D >= (1ll << 31) || 64 * vs[2] + D >= (1ll << 31))
     return fail(MOA_ERR_UNSUPPORTED, "moa_prefill_fwd: k/v token stride too large");
