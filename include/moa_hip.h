@@ -71,7 +71,9 @@ const char* moa_last_error(void);
  * call per (dtype, D) sets a kernel attribute: make one ordinary call per device
  * and (dtype, D) before recording the call into a HIP graph; a recorded call
  * keeps the slot it was recorded with, so replays of ONE graph that overlap each
- * other on a GPU are not supported.
+ * other on a GPU are not supported.  Sizes beyond what the queue arithmetic
+ * covers return MOA_ERR_UNSUPPORTED: B * Hq <= 2^22, B * Hq * ceil(N / 256) <=
+ * 2^25, N <= 2^28.
  */
 int moa_prefill_fwd(const void* q, const void* k, const void* v, void* o,
                     const int64_t* q_strides, const int64_t* k_strides,
