@@ -62,6 +62,20 @@ def test_argument_errors_without_gpu(lib):
         _lib.check(_lib.MOA_ERR_UNSUPPORTED)
 
 
+def test_prefill_size_limits_without_gpu(lib):
+    """Sizes beyond what the prefill work queue's ticket arithmetic covers are refused before anything is
+    launched or looked up on a device (include/moa_hip.h): more than 2^22 (batch, head) pairs, more than
+    2^25 work items, a prompt longer than 2^28."""
+    from moa_amd import _lib
+    I4 = ctypes.c_int64 * 4
+    p = ctypes.c_void_p(0x10000)   # never dereferenced: the call fails on the sizes
+    for B, Hq, N in (((1 << 20), 8, 64), (1 << 16, 8, 1 << 15), (8, 8, 1 << 29)):
+        D = 64
+        st = I4(Hq * N * D, N * D, D, 1)
+        rc = lib.moa_prefill_fwd(p, p, p, p, st, st, st, st, B, Hq, Hq, N, D, p, p, 0.1, _lib.MOA_DTYPE_F16, None)
+        assert rc == _lib.MOA_ERR_UNSUPPORTED and "too many work items" in _lib.last_error(), (B, Hq, N)
+
+
 def test_no_cpu_path():
     from moa_amd import StaticCircularCache, _lib, mixture_of_sparse_attention
     q = torch.zeros(1, 2, 1, 128, dtype=torch.float16)
